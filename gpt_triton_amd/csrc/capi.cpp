@@ -1,0 +1,273 @@
+// The C ABI of libgptmi (declared in include/gptmi.h): argument validation,
+// operand packing for the GEMM, and dispatch to the kernel launchers.
+#include "../../include/gptmi.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+#include "launch.h"
+
+namespace gptmi {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+static int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return GPTMI_ERR_LAUNCH;
+  }
+  return GPTMI_OK;
+}
+
+static bool dtype_ok(int dtype) { return dtype == GPTMI_F32 || dtype == GPTMI_F16; }
+
+static inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// Workspace plan of one GEMM: where the packed weight and (if needed) the
+// packed activations live.
+struct LinearPlan {
+  int Kp;
+  bool pack_x;     // x must be converted / zero padded into the workspace
+  size_t w_off, w_bytes, x_off, x_bytes, total;
+};
+
+static LinearPlan plan_linear(int64_t M, int64_t N, int64_t K, int dtype, int wlayout) {
+  LinearPlan p;
+  p.Kp = (int)round_up(K, 64);
+  p.pack_x = !(dtype == GPTMI_F16 && p.Kp == K);
+  const bool pack_w = !(wlayout == GPTMI_W_NK && dtype == GPTMI_F16 && p.Kp == K);
+  p.w_off = 0;
+  p.w_bytes = pack_w ? (size_t)round_up(N * (int64_t)p.Kp * 2, 256) : 0;
+  p.x_off = p.w_bytes;
+  p.x_bytes = p.pack_x ? (size_t)round_up(M * (int64_t)p.Kp * 2, 256) : 0;
+  p.total = p.w_bytes + p.x_bytes;
+  return p;
+}
+
+// Packs operands as the plan says; returns the A and Bt pointers the GEMM reads.
+static int prepare_operands(const void* x, const void* W, int64_t M, int64_t N, int64_t K,
+                            int dtype, int wlayout, void* workspace, size_t workspace_bytes,
+                            hipStream_t st, const void** A, const void** Bt, int* Kp) {
+  const LinearPlan p = plan_linear(M, N, K, dtype, wlayout);
+  if (p.total > 0) {
+    if (workspace == nullptr || workspace_bytes < p.total) {
+      set_error("linear: workspace of %zu bytes needed, %zu given", p.total,
+                workspace ? workspace_bytes : (size_t)0);
+      return GPTMI_ERR_WORKSPACE;
+    }
+    if (((uintptr_t)workspace & 255) != 0) {
+      set_error("linear: workspace must be 256-byte aligned");
+      return GPTMI_ERR_WORKSPACE;
+    }
+  }
+  const bool f16 = dtype == GPTMI_F16;
+  char* ws = (char*)workspace;
+  if (p.w_bytes) {
+    if (wlayout == GPTMI_W_KN)
+      launch_pack_transpose(W, ws + p.w_off, (int)K, (int)N, p.Kp, f16, st);
+    else
+      launch_pack_rows(W, ws + p.w_off, N, (int)K, p.Kp, f16, st);
+    *Bt = ws + p.w_off;
+  } else {
+    *Bt = W;
+  }
+  if (p.pack_x) {
+    launch_pack_rows(x, ws + p.x_off, M, (int)K, p.Kp, f16, st);
+    *A = ws + p.x_off;
+  } else {
+    *A = x;
+  }
+  *Kp = p.Kp;
+  return GPTMI_OK;
+}
+
+}  // namespace gptmi
+
+using namespace gptmi;
+
+extern "C" {
+
+int gptmi_version(void) { return GPTMI_VERSION; }
+
+const char* gptmi_last_error(void) { return g_err; }
+
+int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out, int64_t B,
+                int64_t L, int64_t V, int64_t P, int64_t H, float p, uint64_t seed,
+                int dtype, void* stream) {
+  (void)seed;
+  if (!ids || !wte || !wpe || !out || B <= 0 || L <= 0 || V <= 0 || P <= 0 || H <= 0 ||
+      !dtype_ok(dtype)) {
+    set_error("embed: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (L > P) {
+    set_error("embed: sequence length %lld exceeds the %lld position rows", (long long)L,
+              (long long)P);
+    return GPTMI_ERR_INVALID;
+  }
+  if (H > (1 << 24)) {
+    set_error("embed: H=%lld too large", (long long)H);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (p != 0.0f) {
+    set_error("embed: dropout (p=%g) is not implemented", (double)p);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  launch_embed(ids, wte, wpe, out, B * L, L, (int)H, dtype == GPTMI_F16, (hipStream_t)stream);
+  return check_launch("embed");
+}
+
+int gptmi_layernorm(const void* x, const void* w, const void* b, void* out, int64_t M,
+                    int64_t H, float eps, int dtype, void* stream) {
+  if (!x || !w || !b || !out || M <= 0 || H <= 0 || !dtype_ok(dtype)) {
+    set_error("layernorm: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (H > 8192) {
+    set_error("layernorm: H=%lld beyond the supported 8192", (long long)H);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  launch_layernorm(x, w, b, out, M, (int)H, eps, dtype == GPTMI_F16, (hipStream_t)stream);
+  return check_launch("layernorm");
+}
+
+int gptmi_softmax(const void* x, void* out, int64_t M, int64_t H, int dtype, void* stream) {
+  if (!x || !out || M <= 0 || H <= 0 || !dtype_ok(dtype)) {
+    set_error("softmax: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (H > 8192) {
+    set_error("softmax: H=%lld beyond the supported 8192", (long long)H);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  launch_softmax(x, out, M, (int)H, dtype == GPTMI_F16, (hipStream_t)stream);
+  return check_launch("softmax");
+}
+
+size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int wlayout) {
+  if (M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype)) return 0;
+  return plan_linear(M, N, K, dtype, wlayout).total;
+}
+
+int gptmi_linear(const void* x, const void* W, const void* bias, const void* residual,
+                 void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
+                 uint64_t seed, int wlayout, void* workspace, size_t workspace_bytes,
+                 int dtype, void* stream) {
+  (void)seed;
+  if (!x || !W || !out || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
+      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK)) {
+    set_error("linear: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (N > (1 << 30) || K > (1 << 30)) {
+    set_error("linear: N or K too large");
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (p != 0.0f) {
+    set_error("linear: dropout (p=%g) is not implemented", (double)p);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const void *A, *Bt;
+  int Kp;
+  int rc = prepare_operands(x, W, M, N, K, dtype, wlayout, workspace, workspace_bytes, st,
+                            &A, &Bt, &Kp);
+  if (rc) return rc;
+  if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) {
+    set_error("linear: x and W must be 16-byte aligned");
+    return GPTMI_ERR_INVALID;
+  }
+  GemmEpilogue ep = {};
+  ep.bias = bias;
+  ep.residual = residual;
+  ep.out = out;
+  ep.gelu = gelu ? 1 : 0;
+  ep.qkv = false;
+  ep.f16 = dtype == GPTMI_F16;
+  rc = launch_gemm(A, Bt, M, (int)N, Kp, ep, st);
+  if (rc) return rc;
+  return check_launch("linear");
+}
+
+int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, void* k,
+                     void* v, int64_t B, int64_t L, int64_t heads, int64_t d, int64_t K,
+                     void* workspace, size_t workspace_bytes, int dtype, void* stream) {
+  if (!x || !W || !q || !k || !v || B <= 0 || L <= 0 || heads <= 0 || d <= 0 || K <= 0 ||
+      !dtype_ok(dtype)) {
+    set_error("linear_qkv: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (d % 8 != 0) {
+    set_error("linear_qkv: head size %lld must be a multiple of 8", (long long)d);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  const int64_t M = B * L, N = 3 * heads * d;
+  if (N > (1 << 30) || K > (1 << 30)) {
+    set_error("linear_qkv: N or K too large");
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const void *A, *Bt;
+  int Kp;
+  int rc = prepare_operands(x, W, M, N, K, dtype, GPTMI_W_KN, workspace, workspace_bytes, st,
+                            &A, &Bt, &Kp);
+  if (rc) return rc;
+  if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) {
+    set_error("linear_qkv: x and W must be 16-byte aligned");
+    return GPTMI_ERR_INVALID;
+  }
+  GemmEpilogue ep = {};
+  ep.bias = bias;
+  ep.q = q;
+  ep.k = k;
+  ep.v = v;
+  ep.L = L;
+  ep.heads = (int)heads;
+  ep.d = (int)d;
+  ep.qkv = true;
+  ep.f16 = dtype == GPTMI_F16;
+  rc = launch_gemm(A, Bt, M, (int)N, Kp, ep, st);
+  if (rc) return rc;
+  return check_launch("linear_qkv");
+}
+
+int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int64_t B,
+                     int64_t N, int64_t Lq, int64_t Lk, int64_t d, float scale, float p,
+                     uint64_t seed, int olayout, int dtype, void* stream) {
+  (void)seed;
+  if (!q || !k || !v || !out || B <= 0 || N <= 0 || Lq <= 0 || Lk <= 0 || d <= 0 ||
+      !dtype_ok(dtype) || (olayout != GPTMI_O_BNLD && olayout != GPTMI_O_BLND)) {
+    set_error("flash_attn: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (Lq != Lk) {
+    set_error("flash_attn: Lq=%lld != Lk=%lld is not supported (the causal mask is "
+              "top-left aligned and padded keys rely on it)",
+              (long long)Lq, (long long)Lk);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (p != 0.0f) {
+    set_error("flash_attn: dropout (p=%g) is not implemented", (double)p);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) ||
+      ((uintptr_t)out & 15)) {
+    set_error("flash_attn: q, k, v and out must be 16-byte aligned");
+    return GPTMI_ERR_INVALID;
+  }
+  int rc = launch_flash_attn(q, k, v, out, B, N, Lq, (int)d, scale, olayout == GPTMI_O_BLND,
+                             dtype == GPTMI_F16, (hipStream_t)stream);
+  if (rc) return rc;
+  return check_launch("flash_attn");
+}
+
+}  // extern "C"

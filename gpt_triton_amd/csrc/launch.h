@@ -1,0 +1,46 @@
+// Host-side launchers implemented by the kernel translation units and called
+// by the C ABI in capi.cpp.  All of them only enqueue work on `st`.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gptmi {
+
+int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
+                 int64_t rows, int64_t L, int H, bool f16, hipStream_t st);
+int launch_layernorm(const void* x, const void* w, const void* b, void* out,
+                     int64_t M, int H, float eps, bool f16, hipStream_t st);
+int launch_softmax(const void* x, void* out, int64_t M, int H, bool f16,
+                   hipStream_t st);
+void launch_pack_rows(const void* src, void* dst, int64_t R, int K, int Kp, bool f16,
+                      hipStream_t st);
+void launch_pack_transpose(const void* src, void* dst, int K, int N, int Kp, bool f16,
+                           hipStream_t st);
+
+// Epilogue description of one GEMM launch: out = gelu?(acc + bias) + residual,
+// stored either as a plain [M][N] matrix or scattered into q/k/v [B][heads][L][d].
+struct GemmEpilogue {
+  const void* bias;      // [N] in the storage dtype, or nullptr
+  const void* residual;  // [M][N] in the storage dtype, or nullptr
+  void* out;             // [M][N] (plain mode)
+  void* q;               // qkv mode: three [B][heads][L][d] tensors
+  void* k;
+  void* v;
+  int64_t L;      // qkv mode: rows per sequence
+  int heads;      // qkv mode
+  int d;          // qkv mode: head size
+  int gelu;       // apply tanh-GELU after the bias
+  bool qkv;       // scatter mode
+  bool f16;       // storage dtype of bias / residual / outputs
+};
+
+// C[M][N] = A[M][Kp] . Bt[N][Kp]^T with fp16 operands (Kp % 64 == 0), fp32
+// accumulation and the fused epilogue above.
+int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
+                const GemmEpilogue& ep, hipStream_t st);
+
+int launch_flash_attn(const void* q, const void* k, const void* v, void* out,
+                      int64_t B, int64_t N, int64_t L, int d, float scale,
+                      bool out_blnd, bool f16, hipStream_t st);
+
+}  // namespace gptmi

@@ -1,0 +1,379 @@
+// Bandwidth-bound row kernels: embedding gather, LayerNorm, row softmax and the
+// operand packers of the GEMM.  One wavefront owns one row; a row is held in
+// registers between its passes so HBM sees one read and one write per element.
+#include "common.h"
+#include "launch.h"
+
+namespace gptmi {
+
+template <typename T> struct Vec;
+template <> struct Vec<_Float16> {
+  static constexpr int N = 8;
+  typedef h8 type;
+};
+template <> struct Vec<float> {
+  static constexpr int N = 4;
+  typedef f4 type;
+};
+
+// ---------------------------------------------------------------------------
+// Embedding gather: out[row,:] = wte[ids[row],:] + wpe[row % L,:]
+// (reference: fused_embeddings_kernel, kernels.py:37-72).  The add is done in
+// fp32 and rounded once, which equals one add in the storage dtype.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void embed_vec_kernel(
+    const int64_t* __restrict__ ids, const T* __restrict__ wte,
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H) {
+  typedef typename Vec<T>::type V;
+  constexpr int VN = Vec<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t tok = ids[row];
+  const int64_t pos = row % L;
+  const V* a = reinterpret_cast<const V*>(wte + tok * H);
+  const V* b = reinterpret_cast<const V*>(wpe + pos * H);
+  V* o = reinterpret_cast<V*>(out + row * H);
+  const int nchunks = H / VN;
+  for (int c = lane; c < nchunks; c += 64) {
+    V va = a[c], vb = b[c], vo;
+#pragma unroll
+    for (int j = 0; j < VN; ++j) vo[j] = (T)((float)va[j] + (float)vb[j]);
+    __builtin_nontemporal_store(vo, o + c);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scalar_kernel(
+    const int64_t* __restrict__ ids, const T* __restrict__ wte,
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t tok = ids[row];
+  const int64_t pos = row % L;
+  for (int c = lane; c < H; c += 64)
+    out[row * H + c] = (T)((float)wte[tok * H + c] + (float)wpe[pos * H + c]);
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm (reference: fused_layer_norm_kernel, kernels.py:104-145): fp32
+// mean, then fp32 centred biased variance, rstd = 1/sqrt(var + eps),
+// z = (x - mean) * rstd * w + b.  CH = 16-byte chunks per lane.
+// ---------------------------------------------------------------------------
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void layernorm_vec_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
+    T* __restrict__ out, int64_t M, int H, float eps) {
+  typedef typename Vec<T>::type V;
+  constexpr int VN = Vec<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int nchunks = H / VN;
+  const V* xr = reinterpret_cast<const V*>(x + row * H);
+  float v[CH][VN];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      V t = __builtin_nontemporal_load(xr + c);
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        v[i][j] = (float)t[j];
+        s += v[i][j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) v[i][j] = 0.f;
+    }
+  }
+  const float mean = wave_sum(s) / (float)H;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    if (lane + i * 64 < nchunks) {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const float d = v[i][j] - mean;
+        q += d * d;
+      }
+    }
+  }
+  const float var = wave_sum(q) / (float)H;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  const V* wv = reinterpret_cast<const V*>(w);
+  const V* bv = reinterpret_cast<const V*>(b);
+  V* o = reinterpret_cast<V*>(out + row * H);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      V tw = wv[c], tb = bv[c], to;
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const float z = (v[i][j] - mean) * rstd;
+        to[j] = (T)(z * (float)tw[j] + (float)tb[j]);
+      }
+      __builtin_nontemporal_store(to, o + c);
+    }
+  }
+}
+
+// Any H (no alignment requirement): the row is re-read from cache per pass.
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_scalar_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
+    T* __restrict__ out, int64_t M, int H, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const T* xr = x + row * H;
+  float s = 0.f;
+  for (int c = lane; c < H; c += 64) s += (float)xr[c];
+  const float mean = wave_sum(s) / (float)H;
+  float q = 0.f;
+  for (int c = lane; c < H; c += 64) {
+    const float d = (float)xr[c] - mean;
+    q += d * d;
+  }
+  const float var = wave_sum(q) / (float)H;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  for (int c = lane; c < H; c += 64) {
+    const float z = ((float)xr[c] - mean) * rstd;
+    out[row * H + c] = (T)(z * (float)w[c] + (float)b[c]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Row softmax: fp32 max, exp(x - max), fp32 sum, divide.
+// ---------------------------------------------------------------------------
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void softmax_vec_kernel(const T* __restrict__ x,
+                                                          T* __restrict__ out,
+                                                          int64_t M, int H) {
+  typedef typename Vec<T>::type V;
+  constexpr int VN = Vec<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int nchunks = H / VN;
+  const V* xr = reinterpret_cast<const V*>(x + row * H);
+  float v[CH][VN];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      V t = __builtin_nontemporal_load(xr + c);
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        v[i][j] = (float)t[j];
+        mx = fmaxf(mx, v[i][j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) v[i][j] = -INFINITY;
+    }
+  }
+  mx = wave_max(mx);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      v[i][j] = __expf(v[i][j] - mx);  // exp(-inf) = 0 for the padding lanes
+      s += v[i][j];
+    }
+  }
+  const float inv = 1.0f / wave_sum(s);
+  V* o = reinterpret_cast<V*>(out + row * H);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      V to;
+#pragma unroll
+      for (int j = 0; j < VN; ++j) to[j] = (T)(v[i][j] * inv);
+      __builtin_nontemporal_store(to, o + c);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_scalar_kernel(const T* __restrict__ x,
+                                                             T* __restrict__ out,
+                                                             int64_t M, int H) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const T* xr = x + row * H;
+  float mx = -INFINITY;
+  for (int c = lane; c < H; c += 64) mx = fmaxf(mx, (float)xr[c]);
+  mx = wave_max(mx);
+  float s = 0.f;
+  for (int c = lane; c < H; c += 64) s += __expf((float)xr[c] - mx);
+  const float inv = 1.0f / wave_sum(s);
+  for (int c = lane; c < H; c += 64)
+    out[row * H + c] = (T)(__expf((float)xr[c] - mx) * inv);
+}
+
+// ---------------------------------------------------------------------------
+// GEMM operand packers.  Both produce fp16 rows of Kp (a multiple of 64)
+// elements, zero filled beyond K, which is the only operand form the MFMA
+// kernel reads.
+//   pack_rows:      src[R][K]  -> dst[R][Kp]   (x, or a weight given as [N][K])
+//   pack_transpose: src[K][N]  -> dst[N][Kp]   (weight given as [K][N])
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void pack_rows_kernel(const T* __restrict__ src,
+                                                        _Float16* __restrict__ dst,
+                                                        int64_t R, int K, int Kp) {
+  const int64_t total = R * (int64_t)Kp;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / Kp;
+    const int k = (int)(i - r * Kp);
+    dst[i] = k < K ? (_Float16)(float)src[r * K + k] : (_Float16)0.f;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pack_transpose_kernel(const T* __restrict__ src,
+                                                             _Float16* __restrict__ dst,
+                                                             int K, int N, int Kp) {
+  __shared__ _Float16 tile[64][65];
+  const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int k = k0 + i, n = n0 + tx;
+    tile[i][tx] = (k < K && n < N) ? (_Float16)(float)src[(int64_t)k * N + n]
+                                   : (_Float16)0.f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int n = n0 + i, k = k0 + tx;
+    if (n < N) dst[(int64_t)n * Kp + k] = tile[tx][i];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host launchers
+// ---------------------------------------------------------------------------
+template <typename T>
+static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
+                          void* out, int64_t rows, int64_t L, int H,
+                          hipStream_t st) {
+  const unsigned grid = (unsigned)((rows + 3) / 4);
+  const bool aligned = (H % Vec<T>::N) == 0 && ((uintptr_t)wte % 16) == 0 &&
+                       ((uintptr_t)wpe % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  if (aligned)
+    hipLaunchKernelGGL(embed_vec_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
+                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+  else
+    hipLaunchKernelGGL(embed_scalar_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
+                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+  return 0;
+}
+
+int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
+                 int64_t rows, int64_t L, int H, bool f16, hipStream_t st) {
+  return f16 ? launch_embed_t<_Float16>(ids, wte, wpe, out, rows, L, H, st)
+             : launch_embed_t<float>(ids, wte, wpe, out, rows, L, H, st);
+}
+
+template <typename T, int CH>
+static void ln_go(const void* x, const void* w, const void* b, void* out, int64_t M,
+                  int H, float eps, hipStream_t st) {
+  hipLaunchKernelGGL((layernorm_vec_kernel<T, CH>), dim3((unsigned)((M + 3) / 4)),
+                     dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
+                     (T*)out, M, H, eps);
+}
+
+template <typename T>
+static int launch_layernorm_t(const void* x, const void* w, const void* b, void* out,
+                              int64_t M, int H, float eps, hipStream_t st) {
+  constexpr int VN = Vec<T>::N;
+  const bool aligned = (H % VN) == 0 && ((uintptr_t)x % 16) == 0 &&
+                       ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0 &&
+                       ((uintptr_t)out % 16) == 0;
+  const int need = aligned ? (H / VN + 63) / 64 : 1 << 30;
+  if (need <= 1) ln_go<T, 1>(x, w, b, out, M, H, eps, st);
+  else if (need <= 2) ln_go<T, 2>(x, w, b, out, M, H, eps, st);
+  else if (need <= 3) ln_go<T, 3>(x, w, b, out, M, H, eps, st);
+  else if (need <= 4) ln_go<T, 4>(x, w, b, out, M, H, eps, st);
+  else if (need <= 8) ln_go<T, 8>(x, w, b, out, M, H, eps, st);
+  else if (need <= 16) ln_go<T, 16>(x, w, b, out, M, H, eps, st);
+  else if (need <= 32) ln_go<T, 32>(x, w, b, out, M, H, eps, st);
+  else
+    hipLaunchKernelGGL(layernorm_scalar_kernel<T>, dim3((unsigned)((M + 3) / 4)),
+                       dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
+                       (T*)out, M, H, eps);
+  return 0;
+}
+
+int launch_layernorm(const void* x, const void* w, const void* b, void* out,
+                     int64_t M, int H, float eps, bool f16, hipStream_t st) {
+  return f16 ? launch_layernorm_t<_Float16>(x, w, b, out, M, H, eps, st)
+             : launch_layernorm_t<float>(x, w, b, out, M, H, eps, st);
+}
+
+template <typename T, int CH>
+static void sm_go(const void* x, void* out, int64_t M, int H, hipStream_t st) {
+  hipLaunchKernelGGL((softmax_vec_kernel<T, CH>), dim3((unsigned)((M + 3) / 4)),
+                     dim3(256), 0, st, (const T*)x, (T*)out, M, H);
+}
+
+template <typename T>
+static int launch_softmax_t(const void* x, void* out, int64_t M, int H,
+                            hipStream_t st) {
+  constexpr int VN = Vec<T>::N;
+  const bool aligned =
+      (H % VN) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int need = aligned ? (H / VN + 63) / 64 : 1 << 30;
+  if (need <= 1) sm_go<T, 1>(x, out, M, H, st);
+  else if (need <= 2) sm_go<T, 2>(x, out, M, H, st);
+  else if (need <= 3) sm_go<T, 3>(x, out, M, H, st);
+  else if (need <= 4) sm_go<T, 4>(x, out, M, H, st);
+  else if (need <= 8) sm_go<T, 8>(x, out, M, H, st);
+  else if (need <= 16) sm_go<T, 16>(x, out, M, H, st);
+  else if (need <= 32) sm_go<T, 32>(x, out, M, H, st);
+  else
+    hipLaunchKernelGGL(softmax_scalar_kernel<T>, dim3((unsigned)((M + 3) / 4)),
+                       dim3(256), 0, st, (const T*)x, (T*)out, M, H);
+  return 0;
+}
+
+int launch_softmax(const void* x, void* out, int64_t M, int H, bool f16,
+                   hipStream_t st) {
+  return f16 ? launch_softmax_t<_Float16>(x, out, M, H, st)
+             : launch_softmax_t<float>(x, out, M, H, st);
+}
+
+void launch_pack_rows(const void* src, void* dst, int64_t R, int K, int Kp, bool f16,
+                      hipStream_t st) {
+  const int64_t total = R * (int64_t)Kp;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (f16)
+    hipLaunchKernelGGL(pack_rows_kernel<_Float16>, dim3((unsigned)blocks), dim3(256),
+                       0, st, (const _Float16*)src, (_Float16*)dst, R, K, Kp);
+  else
+    hipLaunchKernelGGL(pack_rows_kernel<float>, dim3((unsigned)blocks), dim3(256), 0,
+                       st, (const float*)src, (_Float16*)dst, R, K, Kp);
+}
+
+void launch_pack_transpose(const void* src, void* dst, int K, int N, int Kp, bool f16,
+                           hipStream_t st) {
+  dim3 grid((unsigned)(Kp / 64), (unsigned)((N + 63) / 64));
+  if (f16)
+    hipLaunchKernelGGL(pack_transpose_kernel<_Float16>, grid, dim3(256), 0, st,
+                       (const _Float16*)src, (_Float16*)dst, K, N, Kp);
+  else
+    hipLaunchKernelGGL(pack_transpose_kernel<float>, grid, dim3(256), 0, st,
+                       (const float*)src, (_Float16*)dst, K, N, Kp);
+}
+
+}  // namespace gptmi

@@ -1,0 +1,221 @@
+"""Model layer: GPTConfig / FusedGPT / FusedAttention / FusedMLP and the FLOP helpers, with the
+class names, constructor arguments and state_dict keys of the reference's gpt.py so that a
+checkpoint or calling code written for it works unchanged:
+
+    FusedAttention(hidden_size, num_heads, dropout_prob=0.0)     gpt.py:21-67
+    FusedMLP(hidden_size, dropout_prob=0.0)                      gpt.py:70-119
+    GPTConfig                                                    gpt.py:122-129
+    FusedGPT(config)                                             gpt.py:132-196
+    convert_huggingface_to_triton(hf_sd, hf_config)              gpt.py:199-237
+    estimate_days / get_num_parameters / compute_mfu             gpt.py:250-263
+
+Differences, all additive: GPU_TO_FLOPS knows "mi355x"; FusedGPT.forward takes
+`return_logits=True` for the tied LM head the reference leaves commented out
+(gpt.py:159-161, 172-179); `init_synthetic_` draws the N(0, 0.02) benchmark weights;
+`FusedGPT.forward` reads `config.dropout` (the reference reads a `dropout_prob` attribute the
+dataclass does not have, gpt.py:165, and so only works in eval mode).
+"""
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+
+from .kernels import (flash_attention_v1, fused_embeddings, fused_ffn, fused_layer_norm, lm_head,
+                      matmul_and_split_qkv)
+
+# dense fp16/bf16 tensor throughput, FLOP/s
+GPU_TO_FLOPS = {
+    "v100": 130 * 10**12,
+    "a100": 312 * 10**12,
+    "h100": 989 * 10**12,
+    "mi355x": 2500 * 10**12,
+}
+
+
+def _linear_flops(tokens, fan_in, fan_out):
+    # multiply-adds of the product plus the bias add, as gpt.py:62-67 / 113-119 count them
+    return tokens * fan_out * (2 * fan_in) + tokens * fan_out
+
+
+def _norm_flops(tokens, width):
+    return 2 * tokens * width
+
+
+class FusedAttention(nn.Module):
+    """Pre-LN causal self-attention block: x + proj(attention(qkv(LN(x))))."""
+
+    def __init__(self, hidden_size, num_heads, dropout_prob=0.0):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.dropout_prob = dropout_prob
+        h = hidden_size
+        self.layer_norm_weight = nn.Parameter(torch.ones(h))
+        self.layer_norm_bias = nn.Parameter(torch.zeros(h))
+        self.c_attn_weight = nn.Parameter(torch.rand(h, 3 * h))
+        self.c_attn_bias = nn.Parameter(torch.rand(3 * h))
+        self.c_proj_weight = nn.Parameter(torch.rand(h, h))
+        self.c_proj_bias = nn.Parameter(torch.rand(h))
+
+    def forward(self, x):
+        p = self.dropout_prob if self.training else 0.0
+        skip = x
+        y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+        q, k, v = matmul_and_split_qkv(y, self.c_attn_weight.data, self.c_attn_bias.data,
+                                       self.num_heads)
+        # [B, N, L, d] values in a [B, L, N, d] buffer: the head merge below copies nothing
+        y = flash_attention_v1(q, k, v, dropout_prob=p, merged_heads_layout=True)
+        y = y.transpose(1, 2).contiguous().view(skip.shape)
+        return fused_ffn(y, self.c_proj_weight.data, bias=self.c_proj_bias.data, residual=skip,
+                         add_gelu=False, dropout_prob=p)
+
+    def get_fwd_flops(self, num_tokens):
+        h = self.hidden_size
+        return (_norm_flops(num_tokens, h) + _linear_flops(num_tokens, h, 3 * h) +
+                _linear_flops(num_tokens, h, h))
+
+
+class FusedMLP(nn.Module):
+    """Pre-LN feed-forward block: x + ffn2(gelu(ffn1(LN(x)))), inner width 4h."""
+
+    def __init__(self, hidden_size, dropout_prob=0.0):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = 4 * hidden_size
+        self.dropout_prob = dropout_prob
+        h, mid = hidden_size, self.intermediate_size
+        self.layer_norm_weight = nn.Parameter(torch.ones((h,)))
+        self.layer_norm_bias = nn.Parameter(torch.zeros((h,)))
+        self.ffn1_weight = nn.Parameter(torch.rand(h, mid))
+        self.ffn1_bias = nn.Parameter(torch.rand(mid))
+        self.ffn2_weight = nn.Parameter(torch.rand(mid, h))
+        self.ffn2_bias = nn.Parameter(torch.rand(h))
+
+    def forward(self, x):
+        p = self.dropout_prob if self.training else 0.0
+        skip = x
+        y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+        y = fused_ffn(y, self.ffn1_weight.data, bias=self.ffn1_bias.data, residual=None,
+                      add_gelu=True, dropout_prob=p)
+        return fused_ffn(y, self.ffn2_weight.data, bias=self.ffn2_bias.data, residual=skip,
+                         add_gelu=False, dropout_prob=p)
+
+    def get_fwd_flops(self, num_tokens):
+        h, mid = self.hidden_size, self.intermediate_size
+        return (_norm_flops(num_tokens, h) + _linear_flops(num_tokens, h, mid) +
+                _linear_flops(num_tokens, mid, h))
+
+
+@dataclass
+class GPTConfig:
+    vocab_size: int = 50304
+    block_size: int = 512
+    n_layer: int = 12
+    n_head: int = 12
+    n_embd: int = 768
+    dropout: float = 0.1
+
+
+class FusedGPT(nn.Module):
+    """Token + position embeddings, n_layer x (FusedAttention, FusedMLP), final LayerNorm.
+    forward(x) returns the final hidden state [B, L, n_embd], like the reference."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        h = config.n_embd
+        self.wte_weight = nn.Parameter(torch.rand(config.vocab_size, h))
+        self.wpe_weight = nn.Parameter(torch.rand(config.block_size, h))
+        self.blocks = nn.ModuleList([
+            nn.Sequential(FusedAttention(h, config.n_head, dropout_prob=config.dropout),
+                          FusedMLP(h, dropout_prob=config.dropout))
+            for _ in range(config.n_layer)
+        ])
+        self.layer_norm_weight = nn.Parameter(torch.ones((h,)))
+        self.layer_norm_bias = nn.Parameter(torch.zeros((h,)))
+
+    def forward(self, x, return_logits=False):
+        # causal by construction; no attention or padding mask is taken
+        p = self.config.dropout if self.training else 0.0
+        x = fused_embeddings(x, self.wte_weight.data, self.wpe_weight.data, dropout_prob=p)
+        for block in self.blocks:
+            x = block(x)
+        x = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+        if return_logits:
+            return x, lm_head(x, self.wte_weight.data)
+        return x
+
+    def get_fwd_flops(self, num_tokens):
+        cfg = self.config
+        # the embedding lookups are counted as if they were matmuls (gpt.py:182-196)
+        lookups = num_tokens * cfg.n_embd * 2 * (cfg.vocab_size + cfg.block_size)
+        body = sum(m.get_fwd_flops(num_tokens) for blk in self.blocks for m in blk)
+        return body + _norm_flops(num_tokens, cfg.n_embd) + lookups
+
+    @torch.no_grad()
+    def init_synthetic_(self, seed=1337, std=0.02):
+        """Benchmark initialisation: matrices N(0, std), biases 0, LayerNorm (1, 0).  The
+        constructors' U[0,1) values overflow fp16 within a layer."""
+        gen = torch.Generator(device="cpu").manual_seed(seed)
+        for name, prm in self.named_parameters():
+            if "layer_norm_weight" in name:
+                prm.fill_(1.0)
+            elif name.endswith("_bias"):
+                prm.zero_()
+            else:
+                prm.copy_(torch.randn(prm.shape, generator=gen, dtype=torch.float32) * std)
+        return self
+
+
+def convert_huggingface_to_triton(hf_sd, hf_config):
+    """Renames a HuggingFace GPT2Model state dict to FusedGPT's keys.  HF's Conv1D weights are
+    already [in, out], so no tensor is transposed; the causal-mask buffers are dropped."""
+    n_pos = getattr(hf_config, "n_ctx", None) or hf_config.n_positions
+    config = GPTConfig(vocab_size=hf_config.vocab_size, block_size=n_pos,
+                       n_layer=hf_config.n_layer, n_head=hf_config.n_head,
+                       n_embd=hf_config.n_embd, dropout=0.1)
+    rename = {"wte.weight": "wte_weight", "wpe.weight": "wpe_weight",
+              "ln_f.weight": "layer_norm_weight", "ln_f.bias": "layer_norm_bias"}
+    per_layer = {
+        "ln_1.weight": "0.layer_norm_weight", "ln_1.bias": "0.layer_norm_bias",
+        "attn.c_attn.weight": "0.c_attn_weight", "attn.c_attn.bias": "0.c_attn_bias",
+        "attn.c_proj.weight": "0.c_proj_weight", "attn.c_proj.bias": "0.c_proj_bias",
+        "ln_2.weight": "1.layer_norm_weight", "ln_2.bias": "1.layer_norm_bias",
+        "mlp.c_fc.weight": "1.ffn1_weight", "mlp.c_fc.bias": "1.ffn1_bias",
+        "mlp.c_proj.weight": "1.ffn2_weight", "mlp.c_proj.bias": "1.ffn2_bias",
+    }
+    for i in range(config.n_layer):
+        for src, dst in per_layer.items():
+            rename[f"h.{i}.{src}"] = f"blocks.{i}.{dst}"
+    sd = {}
+    for key, tensor in hf_sd.items():
+        if key.endswith("attn.bias") or key.endswith("attn.masked_bias"):
+            continue
+        sd[rename[key]] = tensor
+    return sd, config
+
+
+def convert_hf_and_load_model(model_id, device):
+    """Loads HF GPT-2 weights (a hub name, or a local directory when offline) into a FusedGPT;
+    returns (model, hf_model), both in eval mode on `device`."""
+    from transformers import GPT2Model
+
+    hf_model = GPT2Model.from_pretrained(model_id)
+    state_dict, config = convert_huggingface_to_triton(hf_model.state_dict(), hf_model.config)
+    model = FusedGPT(config)
+    model.load_state_dict(state_dict)
+    return model.to(device).eval(), hf_model.to(device).eval()
+
+
+def estimate_days(flops, mfu=0.45, gpu="h100", num_gpus=1):
+    assert gpu in GPU_TO_FLOPS
+    return flops / (mfu * GPU_TO_FLOPS[gpu] * 3600 * 24 * num_gpus)
+
+
+def get_num_parameters(model):
+    return sum(p.numel() for p in model.parameters())
+
+
+def compute_mfu(flops_per_second, gpu="h100"):
+    assert gpu in GPU_TO_FLOPS
+    return flops_per_second / GPU_TO_FLOPS[gpu]

@@ -1,0 +1,254 @@
+"""Operator layer: the five public functions of the reference's kernels.py, with the same
+names, argument order, defaults, assertions and return shapes, each handing raw device
+pointers to one entry point of libgptmi.so (include/gptmi.h).
+
+    fused_embeddings(x, wte, wpe, dropout_prob=0.0)              kernels.py:75-101
+    fused_layer_norm(x, weight, bias)                            kernels.py:148-164
+    fused_ffn(x, weight, bias=None, residual=None,
+              add_gelu=False, dropout_prob=0.0)                  kernels.py:260-315
+    matmul_and_split_qkv(x, weight, bias, num_heads)             kernels.py:347-367
+    flash_attention_v1(q, k, v, dropout_prob=0.0)                kernels.py:477-525
+
+plus `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:318-342) and
+`lm_head(x, wte)` (the transposed-weight product the reference leaves as a TODO,
+gpt.py:159-161).  Tensors must live on the GPU: there is no CPU path.  dropout_prob > 0
+raises NotImplementedError.
+"""
+import math
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.GPTMI_F32, torch.float16: _lib.GPTMI_F16}
+
+
+def _dtype_code(t, what):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"{what}: dtype {t.dtype} is not supported (float32 and float16 are)")
+
+
+def _on_gpu(*tensors):
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError("gpt_triton_amd operators run on the GPU only; got a tensor on "
+                           f"{dev} (there is no CPU fallback)")
+    for t in tensors[1:]:
+        if t is not None and t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _workspace(nbytes, device):
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+@torch.no_grad()
+def fused_embeddings(x, wte, wpe, dropout_prob=0.0):
+    """dropout(wte[x] + wpe[position]) for token ids x [B, L] -> [B, L, H] in wte's dtype."""
+    assert wte.shape[1] == wpe.shape[1]
+    assert x.is_contiguous()
+    assert wte.is_contiguous()
+    assert wpe.is_contiguous()
+    B, L = x.shape
+    V, H = wte.shape
+    P = wpe.shape[0]
+    if x.dtype != torch.int64:
+        raise TypeError(f"fused_embeddings: token ids must be int64, got {x.dtype}")
+    if wte.dtype != wpe.dtype:
+        raise TypeError("fused_embeddings: wte and wpe must share a dtype")
+    dev = _on_gpu(x, wte, wpe)
+    z = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_embed(x.data_ptr(), wte.data_ptr(), wpe.data_ptr(), z.data_ptr(), B, L, V,
+                             P, H, float(dropout_prob), 1337, _dtype_code(wte, "fused_embeddings"),
+                             _stream())
+    _lib.check(rc, "fused_embeddings")
+    return z.view((B, L, H))
+
+
+@torch.no_grad()
+def fused_layer_norm(x, weight, bias):
+    """LayerNorm over the last dim (eps = 1e-5, biased variance), same shape and dtype as x."""
+    assert x.is_contiguous()
+    assert weight.is_contiguous()
+    assert bias.is_contiguous()
+    assert weight.shape == bias.shape
+    assert x.shape[-1] == weight.shape[0]
+    if not (x.dtype == weight.dtype == bias.dtype):
+        raise TypeError("fused_layer_norm: x, weight and bias must share a dtype")
+    dev = _on_gpu(x, weight, bias)
+    H = x.shape[-1]
+    M = x.numel() // H
+    z = torch.empty(x.shape, device=dev, dtype=x.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_layernorm(x.data_ptr(), weight.data_ptr(), bias.data_ptr(), z.data_ptr(), M,
+                                 H, 1e-5, _dtype_code(x, "fused_layer_norm"), _stream())
+    _lib.check(rc, "fused_layer_norm")
+    return z
+
+
+@torch.no_grad()
+def fused_softmax(x):
+    """softmax over the last dim with fp32 statistics, same shape and dtype as x."""
+    assert x.is_contiguous()
+    dev = _on_gpu(x)
+    H = x.shape[-1]
+    M = x.numel() // H
+    z = torch.empty(x.shape, device=dev, dtype=x.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_softmax(x.data_ptr(), z.data_ptr(), M, H, _dtype_code(x, "fused_softmax"),
+                               _stream())
+    _lib.check(rc, "fused_softmax")
+    return z
+
+
+def _linear(x2d, weight, bias, residual, z, gelu, dropout_prob, wlayout, what):
+    M, K = x2d.shape
+    N = z.shape[1]
+    dev = x2d.device
+    code = _dtype_code(x2d, what)
+    for name, t in (("weight", weight), ("bias", bias), ("residual", residual)):
+        if t is not None and t.dtype != x2d.dtype:
+            raise TypeError(f"{what}: {name} is {t.dtype} but x is {x2d.dtype}")
+    lib = _lib.load()
+    ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, wlayout)
+    ws = _workspace(ws_bytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_linear(x2d.data_ptr(), weight.data_ptr(), _ptr(bias), _ptr(residual),
+                              z.data_ptr(), M, N, K, int(bool(gelu)), float(dropout_prob), 1337,
+                              wlayout, _ptr(ws), ws_bytes, code, _stream())
+    _lib.check(rc, what)
+    return z
+
+
+@torch.no_grad()
+def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False, dropout_prob=0.0):
+    """dropout(gelu?(x @ weight + bias)) + residual; weight is [K, N] (in x out)."""
+    out_shape_0 = x.shape[:-1]
+    x = x.view((-1, x.shape[-1]))
+    M, K = x.shape
+    N = weight.shape[1]
+    dev = _on_gpu(x, weight, bias, residual)
+    z = torch.empty((M, N), device=dev, dtype=x.dtype)
+
+    assert x.is_contiguous()
+    assert weight.is_contiguous()
+    assert x.shape[1] == weight.shape[0]
+    if bias is not None:
+        assert bias.is_contiguous()
+        assert weight.shape[1] == bias.shape[0]
+    if residual is not None:
+        residual = residual.view(z.shape)
+        assert residual.is_contiguous()
+
+    _linear(x, weight, bias, residual, z, add_gelu, dropout_prob, _lib.GPTMI_W_KN, "fused_ffn")
+    return z.view((*out_shape_0, N))
+
+
+@torch.no_grad()
+def lm_head(x, wte):
+    """x @ wte^T for wte [V, H]: logits [*, V] without materialising the transposed weight."""
+    out_shape_0 = x.shape[:-1]
+    x = x.view((-1, x.shape[-1]))
+    assert x.is_contiguous()
+    assert wte.is_contiguous()
+    assert x.shape[1] == wte.shape[1]
+    dev = _on_gpu(x, wte)
+    z = torch.empty((x.shape[0], wte.shape[0]), device=dev, dtype=x.dtype)
+    _linear(x, wte, None, None, z, False, 0.0, _lib.GPTMI_W_NK, "lm_head")
+    return z.view((*out_shape_0, wte.shape[0]))
+
+
+@torch.no_grad()
+def matmul_and_split_qkv(x, weight, bias, num_heads):
+    """x [B, L, h] @ weight [h, 3h] + bias, returned as q, k, v [B, num_heads, L, h/num_heads],
+    each contiguous; the GEMM's store does the head split."""
+    batch_size, seqlen, _ = x.shape
+    assert x.is_contiguous()
+    assert weight.is_contiguous()
+    assert x.shape[2] == weight.shape[0]
+    hidden_size = weight.shape[1]
+    assert hidden_size % 3 == 0, hidden_size
+    hidden_size = hidden_size // 3
+    assert hidden_size % num_heads == 0, (hidden_size, num_heads)
+    head_size = hidden_size // num_heads
+    if bias is not None:
+        assert bias.is_contiguous()
+        assert weight.shape[1] == bias.shape[0]
+    dev = _on_gpu(x, weight, bias)
+    code = _dtype_code(x, "matmul_and_split_qkv")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("matmul_and_split_qkv: x, weight and bias must share a dtype")
+    if head_size % 8 != 0:
+        # the scatter epilogue stores 8-element groups; other head sizes take the plain GEMM
+        y = fused_ffn(x, weight, bias=bias)
+        q, k, v = y.split(hidden_size, dim=2)
+        return tuple(t.view(batch_size, seqlen, num_heads, head_size).transpose(1, 2).contiguous()
+                     for t in (q, k, v))
+    shape = (batch_size, num_heads, seqlen, head_size)
+    q = torch.empty(shape, device=dev, dtype=x.dtype)
+    k = torch.empty(shape, device=dev, dtype=x.dtype)
+    v = torch.empty(shape, device=dev, dtype=x.dtype)
+    lib = _lib.load()
+    M, K, N = batch_size * seqlen, x.shape[2], 3 * hidden_size
+    ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, _lib.GPTMI_W_KN)
+    ws = _workspace(ws_bytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_linear_qkv(x.data_ptr(), weight.data_ptr(), _ptr(bias), q.data_ptr(),
+                                  k.data_ptr(), v.data_ptr(), batch_size, seqlen, num_heads,
+                                  head_size, K, _ptr(ws), ws_bytes, code, _stream())
+    _lib.check(rc, "matmul_and_split_qkv")
+    return q, k, v
+
+
+@torch.no_grad()
+def flash_attention_v1(q, k, v, dropout_prob=0.0, *, merged_heads_layout=False):
+    """Causal softmax(q k^T / sqrt(d)) v for q, k, v [B, N, L, d] -> [B, N, L, d].
+
+    merged_heads_layout=True (an extension; the default is the reference's behaviour)
+    returns the same values as a [B, N, L, d]-shaped view of a [B, L, N, d] buffer, so the
+    caller's `.transpose(1, 2).contiguous()` head merge costs no copy.
+    """
+    assert q.shape[:2] == k.shape[:2]
+    assert q.shape[-1] == k.shape[-1]
+    assert k.shape == v.shape
+    B, N, Lq, H = q.shape
+    Lk = k.shape[2]
+    assert H in {16, 32, 64, 128, 256}
+    assert q.is_contiguous()
+    assert k.is_contiguous()
+    assert v.is_contiguous()
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("flash_attention_v1: q, k and v must share a dtype")
+    dev = _on_gpu(q, k, v)
+    code = _dtype_code(q, "flash_attention_v1")
+    scale = 1 / math.sqrt(H)
+    if merged_heads_layout:
+        buf = torch.empty((B, Lq, N, H), device=dev, dtype=q.dtype)
+        layout = _lib.GPTMI_O_BLND
+    else:
+        buf = torch.empty((B, N, Lq, H), device=dev, dtype=q.dtype)
+        layout = _lib.GPTMI_O_BNLD
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_flash_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), buf.data_ptr(), B, N,
+                                  Lq, Lk, H, scale, float(dropout_prob), 1337, layout, code,
+                                  _stream())
+    _lib.check(rc, "flash_attention_v1")
+    return buf.transpose(1, 2) if merged_heads_layout else buf

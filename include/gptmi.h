@@ -1,0 +1,164 @@
+/*
+ * gptmi.h -- C ABI of libgptmi.so: the GPT-2 forward hot path as hand-written
+ * HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions shared by every entry point
+ *   - all data pointers are DEVICE pointers into memory owned by the caller;
+ *     nothing is allocated, freed or retained by the library;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     every call only enqueues work on it and never synchronises;
+ *   - `dtype` is a gptmi_dtype and names the storage type of the floating
+ *     point tensors of that call (activations, weights and outputs alike);
+ *   - the return value is 0 on success or a negative gptmi_status; the text of
+ *     the most recent failure on the calling thread is gptmi_last_error();
+ *   - the library holds no mutable global state besides that thread-local
+ *     message, so calls from several host threads / streams are independent.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (thevasudevgupta/gpt-triton, file:line).  The reference has no FFI of its
+ * own: its operators are Python functions that launch Triton kernels, and the
+ * entry points below are what those Python functions bind to instead.
+ */
+#ifndef GPTMI_H
+#define GPTMI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPTMI_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef enum gptmi_dtype {
+  GPTMI_F32 = 0, /* IEEE binary32 storage */
+  GPTMI_F16 = 1  /* IEEE binary16 storage, fp32 arithmetic inside kernels */
+} gptmi_dtype;
+
+typedef enum gptmi_status {
+  GPTMI_OK = 0,
+  GPTMI_ERR_INVALID = -1,     /* NULL pointer, non-positive size, bad enum */
+  GPTMI_ERR_UNSUPPORTED = -2, /* valid request the kernels do not implement */
+  GPTMI_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+  GPTMI_ERR_LAUNCH = -4       /* hipGetLastError() after the launch != success */
+} gptmi_status;
+
+/* Layout of the weight operand of gptmi_linear. */
+typedef enum gptmi_wlayout {
+  GPTMI_W_KN = 0, /* W[K][N] row-major: the reference's (and HF Conv1D's) in x out layout */
+  GPTMI_W_NK = 1  /* W[N][K] row-major: out x in, e.g. the tied LM head over wte[V][H] */
+} gptmi_wlayout;
+
+/* Layout of the output of gptmi_flash_attn. */
+typedef enum gptmi_olayout {
+  GPTMI_O_BNLD = 0, /* out[B][N][Lq][d]: what the reference returns */
+  GPTMI_O_BLND = 1  /* out[B][Lq][N][d]: heads already merged, i.e. the result of
+                       out.transpose(1, 2).contiguous() without the copy */
+} gptmi_olayout;
+
+/* Library version (GPTMI_VERSION of the build). */
+int gptmi_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* gptmi_last_error(void);
+
+/*
+ * out[b,l,:] = wte[ids[b,l],:] + wpe[l,:]            (one add in the storage dtype)
+ *
+ * Replaces fused_embeddings(x, wte, wpe, dropout_prob) -> kernels.py:75-101 and
+ * fused_embeddings_kernel -> kernels.py:37-72.
+ *   ids  int64 [B*L]          wte [V][H]     wpe [P][H]     out [B*L][H]
+ * Requires L <= P.  Token ids are NOT range checked on the device (neither does
+ * the reference); the host wrapper may check them.  p must be 0 (dropout is not
+ * implemented: GPTMI_ERR_UNSUPPORTED); seed is accepted for signature stability.
+ */
+int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
+                int64_t B, int64_t L, int64_t V, int64_t P, int64_t H,
+                float p, uint64_t seed, int dtype, void* stream);
+
+/*
+ * out[m,:] = (x[m,:] - mean_m) * rstd_m * w + b, rstd = 1/sqrt(var + eps),
+ * mean and the centred, biased variance in fp32; x is read from HBM once.
+ *
+ * Replaces fused_layer_norm(x, weight, bias) -> kernels.py:148-164 and
+ * fused_layer_norm_kernel -> kernels.py:104-145 (eps = 1e-5 there).
+ *   x, out [M][H]     w, b [H]      1 <= H <= 8192
+ */
+int gptmi_layernorm(const void* x, const void* w, const void* b, void* out,
+                    int64_t M, int64_t H, float eps, int dtype, void* stream);
+
+/*
+ * out[m,:] = softmax(x[m,:]) with fp32 max / sum; x is read from HBM once.
+ *
+ * The reference only sketches this op in a commented-out kernel
+ * (kernels.py:318-342); the contract here is torch.softmax(x.float(), -1).
+ *   x, out [M][H]     1 <= H <= 8192
+ */
+int gptmi_softmax(const void* x, void* out, int64_t M, int64_t H, int dtype,
+                  void* stream);
+
+/*
+ * Bytes of workspace gptmi_linear / gptmi_linear_qkv need for these sizes
+ * (0 if none).  The workspace holds the fp16, K-contiguous, zero-padded copy of
+ * the weight (and of x when x is fp32 or K is not a multiple of 64).
+ */
+size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype,
+                                    int wlayout);
+
+/*
+ * out = gelu?(x @ W + bias) + residual
+ * Operands of the product are rounded to fp16, products and sums are fp32
+ * (MFMA), then in fp32: + bias, tanh-GELU if `gelu`, + residual; one rounding
+ * to the storage dtype at the store.
+ *
+ * Replaces fused_ffn(x, weight, bias, residual, add_gelu, dropout_prob) ->
+ * kernels.py:260-315 and fused_ffn_kernel -> kernels.py:169-257.
+ *   x [M][K]   W [K][N] (GPTMI_W_KN) or [N][K] (GPTMI_W_NK)   bias [N] or NULL
+ *   residual [M][N] or NULL     out [M][N]
+ * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
+ * (may be NULL when that is 0).  p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
+ */
+int gptmi_linear(const void* x, const void* W, const void* bias,
+                 const void* residual, void* out, int64_t M, int64_t N, int64_t K,
+                 int gelu, float p, uint64_t seed, int wlayout, void* workspace,
+                 size_t workspace_bytes, int dtype, void* stream);
+
+/*
+ * y = x @ W + bias with y's 3*heads*d columns split as [q | k | v] and each
+ * third scattered head-major by the GEMM epilogue:
+ *   q[b][n][l][:] = y[b*L + l][n*d : (n+1)*d], k at column offset heads*d,
+ *   v at 2*heads*d.
+ *
+ * Replaces matmul_and_split_qkv(x, weight, bias, num_heads) -> kernels.py:347-367
+ * (fused_ffn followed by split + 3 x view/transpose/contiguous copies).
+ *   x [B*L][K]   W [K][3*heads*d] (GPTMI_W_KN)   bias [3*heads*d] or NULL
+ *   q, k, v [B][heads][L][d]       d a multiple of 8
+ */
+int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
+                     void* k, void* v, int64_t B, int64_t L, int64_t heads,
+                     int64_t d, int64_t K, void* workspace, size_t workspace_bytes,
+                     int dtype, void* stream);
+
+/*
+ * out = softmax(causal(q k^T * scale)) v, mask "key index <= query index".
+ * q, k, v are rounded to fp16; scores, running max, exponentials and the
+ * denominator are fp32; keys are visited in tiles of 64 in ascending order with
+ * the running max updated per tile; P is rounded to fp16 for the P.V product
+ * while the denominator sums the unrounded fp32 P; the final divide is fp32.
+ *
+ * Replaces flash_attention_v1(q, k, v, dropout_prob) -> kernels.py:477-525 and
+ * flash_attention_v1_kernel -> kernels.py:375-474.
+ *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64 or 128    Lq == Lk
+ *   out: [B][N][Lq][d] (GPTMI_O_BNLD) or [B][Lq][N][d] (GPTMI_O_BLND)
+ * p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
+ */
+int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out,
+                     int64_t B, int64_t N, int64_t Lq, int64_t Lk, int64_t d,
+                     float scale, float p, uint64_t seed, int olayout, int dtype,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTMI_H */

@@ -1,0 +1,371 @@
+"""GPU parity: every operator of gpt_triton_amd.kernels (through ctypes -> libgptmi.so) against
+the CPU oracle on the same seeded inputs.  Shapes follow the reference's test.py grids plus
+the GPT-2 sizes; the full BASELINE sizes are checked on sub-samples of independent rows/heads.
+
+Tolerances (stated once, used everywhere):
+  * embedding gather: bit exact;
+  * fp32 storage: max|a-b| <= 1e-4 * max|b|  (north-star "fp32 outputs within 1e-4 relative");
+  * fp16 storage: max|a-b| <= 2 fp16 ulps of max|b| (2 * 2^-10 * max|b|), and for model outputs
+    (hidden state / logits) max|a-b| <= 2e-2 absolute.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gpt2_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+NP = {torch.float32: np.float32, torch.float16: np.float16}
+
+
+@pytest.fixture(scope="module")
+def K(gpu_device):
+    from gpt_triton_amd import kernels
+
+    return kernels
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def check(got, want, dtype, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert np.all(np.isfinite(got)), f"{what}: non-finite output"
+    scale = np.abs(want).max()
+    err = np.abs(got - want).max()
+    tol = (1e-4 if dtype == torch.float32 else 2 * 2.0**-10) * scale
+    assert err <= tol, f"{what}: max|diff| {err:.3e} > {tol:.3e} (max|ref| {scale:.3e})"
+
+
+# ----------------------------------------------------------------------------- embeddings
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("V", [2, 32])
+@pytest.mark.parametrize("H", [32, 128, 256, 33])
+@pytest.mark.parametrize("L,P", [(10, 20), (20, 20)])
+def test_fused_embeddings(K, gpu_device, dtype, V, H, L, P):
+    r = np.random.default_rng(1337)
+    ids = r.integers(0, V, size=(8, L))
+    wte = r.random((V, H)).astype(NP[dtype])
+    wpe = r.random((P, H)).astype(NP[dtype])
+    z = K.fused_embeddings(dev(ids, gpu_device), dev(wte, gpu_device), dev(wpe, gpu_device))
+    assert z.shape == (8, L, H) and z.dtype == dtype
+    assert np.array_equal(host(z), O.fused_embeddings(ids, wte, wpe))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_fused_embeddings_gpt2_shape(K, gpu_device, dtype):
+    r = np.random.default_rng(7)
+    V, H, P, B, L = 50257, 768, 1024, 16, 300
+    ids = r.integers(0, V, size=(B, L))
+    ids[0, 0], ids[0, 1] = 0, V - 1
+    wte = (0.02 * r.standard_normal((V, H))).astype(NP[dtype])
+    wpe = (0.02 * r.standard_normal((P, H))).astype(NP[dtype])
+    z = K.fused_embeddings(dev(ids, gpu_device), dev(wte, gpu_device), dev(wpe, gpu_device))
+    assert np.array_equal(host(z), O.fused_embeddings(ids, wte, wpe))
+
+
+# ----------------------------------------------------------------------------- layer norm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M", [249, 32])
+@pytest.mark.parametrize("Kdim", [123, 128, 64, 768, 1600, 3072])
+def test_fused_layer_norm(K, gpu_device, dtype, M, Kdim):
+    r = np.random.default_rng(1337)
+    x = r.random((M, Kdim)).astype(NP[dtype])
+    w = (1 + 0.1 * r.standard_normal(Kdim)).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(Kdim)).astype(NP[dtype])
+    z = K.fused_layer_norm(dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device))
+    assert z.shape == x.shape and z.dtype == dtype
+    check(host(z), O.fused_layer_norm(x, w, b), dtype, "layer_norm")
+
+
+def test_fused_layer_norm_keeps_leading_dims(K, gpu_device):
+    r = np.random.default_rng(3)
+    x = r.standard_normal((2, 5, 768)).astype(np.float32)
+    w, b = np.ones(768, np.float32), np.zeros(768, np.float32)
+    z = K.fused_layer_norm(dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device))
+    assert z.shape == (2, 5, 768)
+    check(host(z), O.fused_layer_norm(x, w, b), torch.float32)
+
+
+# ----------------------------------------------------------------------------- softmax
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,H", [(33, 768), (5, 123), (17, 64), (9, 2048)])
+def test_fused_softmax(K, gpu_device, dtype, M, H):
+    r = np.random.default_rng(11)
+    x = (3 * r.standard_normal((M, H))).astype(NP[dtype])
+    z = K.fused_softmax(dev(x, gpu_device))
+    check(host(z), O.softmax_rows(x), dtype, "softmax")
+
+
+# ----------------------------------------------------------------------------- fused_ffn
+def ffn_inputs(M, N, Kd, dtype, seed=1337, gaussian=False):
+    r = np.random.default_rng(seed)
+    if gaussian:
+        x = r.standard_normal((M, Kd))
+        w = 0.02 * r.standard_normal((Kd, N))
+        b = 0.02 * r.standard_normal(N)
+        res = r.standard_normal((M, N))
+    else:  # U[0,1) like test.py:17-25
+        x, w, b, res = r.random((M, Kd)), r.random((Kd, N)), r.random(N), r.random((M, N))
+    t = NP[dtype]
+    return x.astype(t), w.astype(t), b.astype(t), res.astype(t)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd", [(128, 128, 256), (199, 129, 129), (61, 31, 23)])
+@pytest.mark.parametrize("add_gelu", [True, False])
+@pytest.mark.parametrize("add_bias", [True, False])
+def test_fused_ffn_reference_grid(K, gpu_device, dtype, M, N, Kd, add_gelu, add_bias):
+    x, w, b, res = ffn_inputs(M, N, Kd, dtype)
+    if dtype == torch.float16:
+        w = (w / Kd).astype(np.float16)  # keep sums of K products inside fp16 range
+    if not add_bias:
+        b = None
+    if Kd != N:
+        res = None
+    z = K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device),
+                    bias=None if b is None else dev(b, gpu_device),
+                    residual=None if res is None else dev(res, gpu_device), add_gelu=add_gelu)
+    assert z.shape == (M, N) and z.dtype == dtype
+    check(host(z), O.fused_ffn(x, w, bias=b, residual=res, add_gelu=add_gelu), dtype, "ffn")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd,gelu,use_res", [
+    (4096, 3072, 768, True, False),   # ffn1 shape, big-tile kernel
+    (4096, 768, 3072, False, True),   # ffn2 shape + residual
+    (2500, 2304, 768, False, False),  # ragged M on the big-tile kernel
+    (2100, 1000, 320, True, True),    # ragged M and N
+    (300, 768, 768, False, True),     # small-tile kernel
+])
+def test_fused_ffn_gpt2_shapes(K, gpu_device, dtype, M, N, Kd, gelu, use_res):
+    x, w, b, res = ffn_inputs(M, N, Kd, dtype, seed=5, gaussian=True)
+    res = res if use_res else None
+    z = K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device),
+                    residual=None if res is None else dev(res, gpu_device), add_gelu=gelu)
+    check(host(z), O.fused_ffn(x, w, bias=b, residual=res, add_gelu=gelu), dtype, "ffn")
+
+
+def test_fused_ffn_leading_dims_and_residual_view(K, gpu_device):
+    x, w, b, res = ffn_inputs(6 * 50, 128, 128, torch.float32, seed=9, gaussian=True)
+    z = K.fused_ffn(dev(x.reshape(6, 50, 128), gpu_device), dev(w, gpu_device),
+                    bias=dev(b, gpu_device), residual=dev(res.reshape(6, 50, 128), gpu_device))
+    assert z.shape == (6, 50, 128)
+    check(host(z).reshape(300, 128), O.fused_ffn(x, w, bias=b, residual=res), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_lm_head_transposed_weight(K, gpu_device, dtype):
+    r = np.random.default_rng(21)
+    x = r.standard_normal((130, 768)).astype(NP[dtype])
+    wte = (0.02 * r.standard_normal((50257, 768))).astype(NP[dtype])
+    z = K.lm_head(dev(x, gpu_device), dev(wte, gpu_device))
+    assert z.shape == (130, 50257)
+    check(host(z), O.fused_ffn(x, np.ascontiguousarray(wte.T)), dtype, "lm_head")
+
+
+# ----------------------------------------------------------------------------- qkv split
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("B,L,heads,d", [(2, 77, 12, 64), (3, 50, 5, 64), (2, 40, 3, 20)])
+def test_matmul_and_split_qkv(K, gpu_device, dtype, B, L, heads, d):
+    r = np.random.default_rng(13)
+    h = heads * d
+    x = r.standard_normal((B, L, h)).astype(NP[dtype])
+    w = (0.05 * r.standard_normal((h, 3 * h))).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(3 * h)).astype(NP[dtype])
+    q, k, v = K.matmul_and_split_qkv(dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device),
+                                     heads)
+    wq, wk, wv = O.matmul_and_split_qkv(x, w, b, heads)
+    for got, want in ((q, wq), (k, wk), (v, wv)):
+        assert got.shape == (B, heads, L, d) and got.is_contiguous()
+        check(host(got), want, dtype, "qkv")
+
+
+# ----------------------------------------------------------------------------- attention
+def attn_inputs(B, N, L, D, dtype, gaussian, seed=1337):
+    r = np.random.default_rng(seed)
+    f = r.standard_normal if gaussian else r.random
+    return tuple(f((B, N, L, D)).astype(NP[dtype]) for _ in range(3))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("B,N", [(3, 9), (2, 7)])
+@pytest.mark.parametrize("L", [199, 128, 63])
+@pytest.mark.parametrize("D", [64, 128])
+def test_flash_attention_reference_grid(K, gpu_device, dtype, B, N, L, D):
+    q, k, v = attn_inputs(B, N, L, D, dtype, gaussian=False)
+    z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+    assert z.shape == (B, N, L, D) and z.dtype == dtype and z.is_contiguous()
+    check(host(z), O.flash_attention_v1(q, k, v), dtype, "attention")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("L", [1, 2, 31, 64, 65, 300, 513])
+def test_flash_attention_gaussian_lengths(K, gpu_device, dtype, L):
+    q, k, v = attn_inputs(2, 12, L, 64, dtype, gaussian=True, seed=L)
+    z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+    check(host(z), O.flash_attention_v1(q, k, v), dtype, f"attention L={L}")
+    # row 0 sees key 0 only
+    assert np.array_equal(host(z)[:, :, 0].astype(np.float32),
+                          v[:, :, 0].astype(np.float16).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_flash_attention_merged_heads_layout(K, gpu_device, dtype):
+    q, k, v = attn_inputs(3, 5, 130, 64, dtype, gaussian=True, seed=3)
+    args = [dev(t, gpu_device) for t in (q, k, v)]
+    a = K.flash_attention_v1(*args)
+    b = K.flash_attention_v1(*args, merged_heads_layout=True)
+    assert b.shape == a.shape
+    assert b.transpose(1, 2).is_contiguous()  # the model's head merge is then a no-op
+    assert torch.equal(a, b)
+
+
+def test_flash_attention_is_causal(K, gpu_device):
+    q, k, v = attn_inputs(1, 2, 200, 64, torch.float32, gaussian=True, seed=17)
+    a = K.flash_attention_v1(*[dev(t, gpu_device) for t in (q, k, v)])
+    k[:, :, 150:] += 1.0
+    v[:, :, 150:] -= 2.0
+    b = K.flash_attention_v1(*[dev(t, gpu_device) for t in (q, k, v)])
+    assert torch.equal(a[:, :, :150], b[:, :, :150])
+    assert not torch.equal(a[:, :, 150:], b[:, :, 150:])
+
+
+# ----------------------------------------------------------------------------- error behaviour
+def test_operator_errors(K, gpu_device):
+    x = torch.zeros((4, 64), device=gpu_device)
+    w = torch.zeros((64, 32), device=gpu_device)
+    with pytest.raises(AssertionError):
+        K.fused_ffn(x.t()[:, :4].t()[:, ::2], w)  # non-contiguous x
+    with pytest.raises(AssertionError):
+        K.fused_ffn(x, torch.zeros((32, 64), device=gpu_device).t())  # non-contiguous weight
+    with pytest.raises(AssertionError):
+        K.fused_ffn(x, torch.zeros((63, 32), device=gpu_device))  # K mismatch
+    with pytest.raises(AssertionError):
+        K.fused_layer_norm(x, torch.ones(63, device=gpu_device), torch.zeros(63, device=gpu_device))
+    with pytest.raises(AssertionError):
+        q = torch.zeros((1, 1, 8, 48), device=gpu_device)  # head size not in the allowed set
+        K.flash_attention_v1(q, q, q)
+    with pytest.raises(NotImplementedError):
+        K.fused_ffn(x, w, dropout_prob=0.1)
+    with pytest.raises(TypeError):
+        K.fused_ffn(x.double(), w.double())
+
+
+# ----------------------------------------------------------------------------- whole model
+def load_params(model, params, dtype, device):
+    sd = {k: torch.from_numpy(np.asarray(v)).to(dtype) for k, v in params.items()}
+    model.load_state_dict(sd)
+    return model.to(device=device, dtype=dtype).eval()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_gpt2_small_forward(gpu_device, dtype):
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig
+
+    cfg = dict(n_layer=3, n_head=4, n_embd=256, vocab_size=1000, block_size=128)
+    params = O.synthetic_params(**cfg, seed=3, std=0.05, dtype=NP[dtype])
+    ids = O.synthetic_ids(3, 100, cfg["vocab_size"], seed=3)
+    model = load_params(FusedGPT(GPTConfig(dropout=0.1, **cfg)), params, dtype, gpu_device)
+    hidden, logits = model(dev(ids, gpu_device), return_logits=True)
+    want_h, want_l = O.gpt2_forward(params, ids, cfg["n_head"], lm_head=True)
+    if dtype == torch.float32:
+        check(host(hidden), want_h, dtype, "hidden")
+        check(host(logits), want_l, dtype, "logits")
+    else:
+        assert np.abs(host(hidden).astype(np.float64) - want_h).max() <= 2e-2
+        assert np.abs(host(logits).astype(np.float64) - want_l).max() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_gpt2_124m_config0(gpu_device, dtype):
+    """BASELINE config 0: 12 x 768 x 12 heads, vocab 50257, 1024 positions, N(0, 0.02)
+    weights, batch 2 x seqlen 64; hidden state and logits [2, 64, 50257]."""
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig
+
+    cfg = dict(n_layer=12, n_head=12, n_embd=768, vocab_size=50257, block_size=1024)
+    params = O.synthetic_params(**cfg, seed=1337, dtype=NP[dtype])
+    ids = O.synthetic_ids(2, 64, cfg["vocab_size"], seed=1337)
+    model = load_params(FusedGPT(GPTConfig(dropout=0.1, **cfg)), params, dtype, gpu_device)
+    hidden, logits = model(dev(ids, gpu_device), return_logits=True)
+    assert hidden.shape == (2, 64, 768) and logits.shape == (2, 64, 50257)
+    want_h, want_l = O.gpt2_forward(params, ids, cfg["n_head"], lm_head=True)
+    if dtype == torch.float32:
+        check(host(hidden), want_h, dtype, "hidden")
+        check(host(logits), want_l, dtype, "logits")
+    else:
+        assert np.abs(host(hidden).astype(np.float64) - want_h).max() <= 2e-2
+        assert np.abs(host(logits).astype(np.float64) - want_l).max() <= 2e-2
+
+
+# ----------------------------------------------------------------------------- BASELINE sizes
+def test_full_size_ffn_rows(K, gpu_device):
+    """BASELINE config 1: X [153600, 768] fp16 @ W [768, 3072] + b -> GELU, then the down
+    projection [153600, 3072] @ [3072, 768] + b (+ residual).  Rows of a GEMM are independent,
+    so a random sample of rows is compared with the oracle run on those rows alone."""
+    g = torch.Generator(device="cpu").manual_seed(1)
+    M = 153600
+    x = torch.randn((M, 768), generator=g).half()
+    w1 = (0.02 * torch.randn((768, 3072), generator=g)).half()
+    b1 = (0.02 * torch.randn(3072, generator=g)).half()
+    w2 = (0.02 * torch.randn((3072, 768), generator=g)).half()
+    b2 = (0.02 * torch.randn(768, generator=g)).half()
+    xd = x.to(gpu_device)
+    y = K.fused_ffn(xd, w1.to(gpu_device), bias=b1.to(gpu_device), add_gelu=True)
+    z = K.fused_ffn(y, w2.to(gpu_device), bias=b2.to(gpu_device), residual=xd)
+    rows = torch.cat([torch.tensor([0, 1, 255, 256, M - 257, M - 1]),
+                      torch.randint(0, M, (250,), generator=g)])
+    y_s, z_s = y[rows.to(gpu_device)].cpu().numpy(), z[rows.to(gpu_device)].cpu().numpy()
+    xs = x[rows].numpy()
+    want_y = O.fused_ffn(xs, w1.numpy(), bias=b1.numpy(), add_gelu=True)
+    check(y_s, want_y, torch.float16, "ffn1 full size")
+    want_z = O.fused_ffn(y_s, w2.numpy(), bias=b2.numpy(), residual=xs)
+    check(z_s, want_z, torch.float16, "ffn2 full size")
+    # linearity in the rows: a checksum of every output row block catches unwritten tiles
+    assert torch.isfinite(y).all() and torch.isfinite(z).all()
+    assert (y.float().abs().sum(dim=1) > 0).all()
+
+
+def test_full_size_attention_heads(K, gpu_device):
+    """BASELINE config 2: q, k, v [512, 12, 300, 64] fp16; (batch, head) pairs are independent."""
+    g = torch.Generator(device="cpu").manual_seed(2)
+    B, N, L, D = 512, 12, 300, 64
+    q, k, v = (torch.randn((B, N, L, D), generator=g).half() for _ in range(3))
+    z = K.flash_attention_v1(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))
+    assert torch.isfinite(z).all()
+    for b, n in [(0, 0), (511, 11), (17, 5), (300, 7)]:
+        want = O.flash_attention_v1(q[b:b + 1, n:n + 1].numpy(), k[b:b + 1, n:n + 1].numpy(),
+                                    v[b:b + 1, n:n + 1].numpy())
+        check(z[b:b + 1, n:n + 1].cpu().numpy(), want, torch.float16, f"attention ({b},{n})")
+    # row 0 of every head is v[:, :, 0] exactly
+    assert torch.equal(z[:, :, 0].cpu(), v[:, :, 0])
+
+
+def test_full_size_rowops(K, gpu_device):
+    """BASELINE config 2: LayerNorm and softmax on [153600, 768] fp16."""
+    g = torch.Generator(device="cpu").manual_seed(3)
+    M, H = 153600, 768
+    x = torch.randn((M, H), generator=g).half()
+    w = (1 + 0.02 * torch.randn(H, generator=g)).half()
+    b = (0.02 * torch.randn(H, generator=g)).half()
+    xd = x.to(gpu_device)
+    ln = K.fused_layer_norm(xd, w.to(gpu_device), b.to(gpu_device))
+    sm = K.fused_softmax(xd)
+    rows = torch.cat([torch.tensor([0, 1, 2, 3, M - 4, M - 1]), torch.randint(0, M, (300,), generator=g)])
+    xs = x[rows].numpy()
+    check(ln[rows.to(gpu_device)].cpu().numpy(), O.fused_layer_norm(xs, w.numpy(), b.numpy()),
+          torch.float16, "layer_norm full size")
+    check(sm[rows.to(gpu_device)].cpu().numpy(), O.softmax_rows(xs), torch.float16,
+          "softmax full size")
+    # every softmax row sums to one (fp16 rounding of 768 terms)
+    assert (sm.float().sum(dim=1) - 1).abs().max() < 2e-3

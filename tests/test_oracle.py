@@ -1,0 +1,323 @@
+"""Pins the CPU oracle (oracle/gpt2_oracle.py) against things it did not come from: library
+routines, fp64 closed forms, invariants and special cases chosen so that a dropped term, a
+wrong sign/index or a transposed operand fails.  No GPU involved."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gpt2_oracle as O
+
+
+def rng(seed=1337):
+    return np.random.default_rng(seed)
+
+
+def h16(a):
+    return a.astype(np.float16).astype(np.float64)
+
+
+# ----------------------------------------------------------------------------- embeddings
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("V,H,L,P", [(2, 32, 10, 20), (32, 128, 20, 20), (32, 256, 10, 20)])
+def test_embeddings_closed_form(dtype, V, H, L, P):
+    # the reference's own oracle, test.py:41
+    r = rng()
+    ids = r.integers(0, V, size=(8, L))
+    wte = r.random((V, H)).astype(dtype)
+    wpe = r.random((P, H)).astype(dtype)
+    want = torch.from_numpy(wte)[torch.from_numpy(ids)] + torch.from_numpy(wpe)[torch.arange(L)][None]
+    got = O.fused_embeddings(ids, wte, wpe)
+    assert got.dtype == dtype
+    assert np.array_equal(got, want.numpy())
+
+
+def test_embeddings_position_is_row_mod_L():
+    # wte = 0 isolates the position term: out[b, l] must be wpe[l] for every b
+    ids = np.zeros((3, 5), dtype=np.int64)
+    wte = np.zeros((1, 4), np.float32)
+    wpe = np.arange(28, dtype=np.float32).reshape(7, 4)
+    got = O.fused_embeddings(ids, wte, wpe)
+    for b in range(3):
+        assert np.array_equal(got[b], wpe[:5])
+
+
+# ----------------------------------------------------------------------------- layer norm
+@pytest.mark.parametrize("M,K", [(249, 123), (32, 128), (249, 64), (7, 768)])
+def test_layer_norm_vs_torch_fp64(M, K):
+    r = rng()
+    x = r.random((M, K)).astype(np.float32)  # U[0,1) like test.py:17-25
+    w = (1 + 0.1 * r.standard_normal(K)).astype(np.float32)
+    b = (0.1 * r.standard_normal(K)).astype(np.float32)
+    want = torch.nn.functional.layer_norm(torch.from_numpy(x).double(), (K,),
+                                          torch.from_numpy(w).double(),
+                                          torch.from_numpy(b).double(), 1e-5).numpy()
+    got = O.fused_layer_norm(x, w, b)
+    assert np.abs(got - want).max() < 2e-6
+
+
+def test_layer_norm_invariants():
+    r = rng(3)
+    x = (5 + 3 * r.standard_normal((16, 96))).astype(np.float32)
+    one, zero = np.ones(96, np.float32), np.zeros(96, np.float32)
+    y = O.fused_layer_norm(x, one, zero)
+    assert np.abs(y.mean(axis=1)).max() < 1e-6
+    assert np.abs(y.var(axis=1) - 1).max() < 1e-4  # biased variance; eps makes it < 1
+    # shift invariance and the eps term: a constant row normalises to exactly beta
+    c = np.full((2, 96), 7.25, np.float32)
+    assert np.array_equal(O.fused_layer_norm(c, one, zero + 0.5), np.full((2, 96), 0.5, np.float32))
+    # eps = 1e-5 matters for tiny-variance rows: var = 1e-6 -> scale 1/sqrt(1.1e-5)
+    t = np.tile(np.array([1e-3, -1e-3], np.float32), 48)[None]
+    got = O.fused_layer_norm(t, one, zero)[0, 0]
+    assert abs(got - 1e-3 / math.sqrt(1e-6 + 1e-5)) < 1e-6
+
+
+def test_layer_norm_fp16_storage():
+    r = rng(5)
+    x = r.standard_normal((9, 768)).astype(np.float16)
+    w = (1 + 0.02 * r.standard_normal(768)).astype(np.float16)
+    b = (0.02 * r.standard_normal(768)).astype(np.float16)
+    want = torch.nn.functional.layer_norm(torch.from_numpy(x).double(), (768,),
+                                          torch.from_numpy(w).double(),
+                                          torch.from_numpy(b).double(), 1e-5)
+    got = O.fused_layer_norm(x, w, b)
+    assert got.dtype == np.float16
+    # one fp16 rounding of the fp64 answer
+    assert np.abs(got.astype(np.float64) - want.numpy()).max() <= 2.0**-11 * 8
+
+
+# ----------------------------------------------------------------------------- GELU
+def test_gelu_vs_torch_tanh_form():
+    x = np.linspace(-12, 12, 4801).astype(np.float32)
+    want = torch.nn.functional.gelu(torch.from_numpy(x).double(), approximate="tanh").numpy()
+    got = O.gelu_new(x)
+    assert np.abs(got - want).max() < 2e-6
+    big = O.gelu_new(np.array([-1e4, -100.0, 100.0, 1e4], np.float32))
+    assert np.array_equal(big, np.array([0.0, 0.0, 100.0, 1e4], np.float32)) or \
+        np.allclose(big, [0.0, 0.0, 100.0, 1e4])
+    assert np.all(np.isfinite(big))
+
+
+# ----------------------------------------------------------------------------- fused_ffn
+def ffn_fp64(x, w, b=None, r=None, gelu=False):
+    z = h16(x) @ h16(w)
+    if b is not None:
+        z = z + b.astype(np.float64)
+    if gelu:
+        z = torch.nn.functional.gelu(torch.from_numpy(z), approximate="tanh").numpy()
+    if r is not None:
+        z = z + r.astype(np.float64)
+    return z
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 256), (199, 129, 129), (61, 31, 23)])
+@pytest.mark.parametrize("gelu", [True, False])
+@pytest.mark.parametrize("bias", [True, False])
+def test_ffn_vs_fp64(M, N, K, gelu, bias):
+    # shapes and U[0,1) inputs of test.py:62-87; residual only when K == N (test.py:23-24)
+    r = rng()
+    x = r.random((M, K)).astype(np.float32)
+    w = r.random((K, N)).astype(np.float32)
+    b = r.random(N).astype(np.float32) if bias else None
+    res = r.random((M, N)).astype(np.float32) if K == N else None
+    want = ffn_fp64(x, w, b, res, gelu)
+    got = O.fused_ffn(x, w, bias=b, residual=res, add_gelu=gelu)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+
+
+def test_ffn_rounds_operands_to_fp16_not_fp32():
+    # a true-fp32 product differs from the fp16-operand product by ~4e-4 relative
+    r = rng(11)
+    x = r.standard_normal((64, 512)).astype(np.float32)
+    w = (0.02 * r.standard_normal((512, 64))).astype(np.float32)
+    got = O.fused_ffn(x, w).astype(np.float64)
+    rounded = h16(x) @ h16(w)
+    exact = x.astype(np.float64) @ w.astype(np.float64)
+    assert np.abs(got - rounded).max() < 1e-5
+    assert np.abs(got - exact).max() > 1e-4
+
+
+def test_ffn_is_not_transposed_and_epilogue_order():
+    # asymmetric one-hot operands: z[m, n] = x[m, :] . w[:, n]
+    x = np.zeros((2, 3), np.float32)
+    w = np.zeros((3, 4), np.float32)
+    x[1, 2] = 2.0
+    w[2, 3] = 3.0
+    z = O.fused_ffn(x, w)
+    want = np.zeros((2, 4), np.float32)
+    want[1, 3] = 6.0
+    assert np.array_equal(z, want)
+    # order bias -> gelu -> residual: gelu(0 + b) + r, not gelu(0 + b + r)
+    b = np.full(4, -3.0, np.float32)
+    r = np.full((2, 4), 10.0, np.float32)
+    z = O.fused_ffn(np.zeros((2, 3), np.float32), w, bias=b, residual=r, add_gelu=True)
+    g = float(torch.nn.functional.gelu(torch.tensor(-3.0, dtype=torch.float64), approximate="tanh"))
+    assert np.allclose(z, 10.0 + g, atol=1e-6)
+
+
+def test_ffn_fp16_storage_rounds_once():
+    r = rng(13)
+    x = r.standard_normal((32, 768)).astype(np.float16)
+    w = (0.02 * r.standard_normal((768, 96))).astype(np.float16)
+    b = (0.02 * r.standard_normal(96)).astype(np.float16)
+    want = ffn_fp64(x, w, b, None, True)
+    got = O.fused_ffn(x, w, bias=b, add_gelu=True)
+    assert got.dtype == np.float16
+    assert np.abs(got.astype(np.float64) - want).max() <= 2.0**-11 * np.abs(want).max() + 1e-6
+
+
+# ----------------------------------------------------------------------------- qkv split
+def test_split_qkv_is_the_index_identity():
+    r = rng(17)
+    B, L, heads, d = 2, 5, 3, 8
+    h = heads * d
+    x = r.standard_normal((B, L, h)).astype(np.float32)
+    w = (0.1 * r.standard_normal((h, 3 * h))).astype(np.float32)
+    b = r.standard_normal(3 * h).astype(np.float32)
+    y = O.fused_ffn(x, w, bias=b)
+    q, k, v = O.matmul_and_split_qkv(x, w, b, heads)
+    assert q.shape == (B, heads, L, d)
+    for bb in range(B):
+        for n in range(heads):
+            for l in range(L):
+                assert np.array_equal(q[bb, n, l], y[bb, l, n * d:(n + 1) * d])
+                assert np.array_equal(k[bb, n, l], y[bb, l, h + n * d:h + (n + 1) * d])
+                assert np.array_equal(v[bb, n, l], y[bb, l, 2 * h + n * d:2 * h + (n + 1) * d])
+
+
+# ----------------------------------------------------------------------------- attention
+def attention_fp64(q, k, v):
+    # test.py:98-106 on the fp16-rounded operands
+    B, N, L, D = q.shape
+    q, k, v = (torch.from_numpy(h16(t)).view(B * N, L, D) for t in (q, k, v))
+    s = (q @ k.transpose(1, 2)) / math.sqrt(D)
+    mask = torch.tril(torch.ones((L, L), dtype=torch.bool))
+    s = torch.where(mask, s, float("-inf"))
+    return (s.softmax(-1) @ v).view(B, N, L, D).numpy()
+
+
+@pytest.mark.parametrize("B,N", [(3, 9), (2, 7)])
+@pytest.mark.parametrize("L", [199, 128, 63])
+@pytest.mark.parametrize("D", [64, 128])
+def test_attention_vs_textbook(B, N, L, D):
+    r = rng()
+    q, k, v = (r.random((B, N, L, D)).astype(np.float32) for _ in range(3))
+    want = attention_fp64(q, k, v)
+    got = O.flash_attention_v1(q, k, v)
+    # the only modelled difference is the fp16 rounding of P (<= 2^-11 relative per weight)
+    assert np.abs(got - want).max() <= 2.0**-11 * np.abs(want).max()
+
+
+def test_attention_gaussian_inputs_and_invariants():
+    r = rng(23)
+    B, N, L, D = 2, 3, 150, 64
+    q, k, v = (r.standard_normal((B, N, L, D)).astype(np.float32) for _ in range(3))
+    got = O.flash_attention_v1(q, k, v)
+    want = attention_fp64(q, k, v)
+    assert np.abs(got - want).max() <= 2.0**-10 * np.abs(v).max()
+    # row 0 attends to key 0 only -> exactly v16[0]
+    assert np.array_equal(got[:, :, 0], v.astype(np.float16).astype(np.float32)[:, :, 0])
+    # every output is a convex combination of the visible value rows
+    v16 = v.astype(np.float16).astype(np.float32)
+    for l in (1, 7, 64, 149):
+        lo, hi = v16[:, :, :l + 1].min(axis=2), v16[:, :, :l + 1].max(axis=2)
+        assert np.all(got[:, :, l] >= lo - 1e-3) and np.all(got[:, :, l] <= hi + 1e-3)
+    # causality: changing a future key/value must not change earlier rows
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, 100:] += 1.0
+    v2[:, :, 100:] -= 2.0
+    got2 = O.flash_attention_v1(q, k2, v2)
+    assert np.array_equal(got[:, :, :100], got2[:, :, :100])
+    assert not np.array_equal(got[:, :, 100:], got2[:, :, 100:])
+
+
+def test_attention_single_tile_equals_plain_softmax():
+    # L <= 64: one key tile, no rescaling; P = exp(S - rowmax) rounded to fp16, denominator
+    # from the unrounded P.  Restated here with plain loops, not with the oracle's code path.
+    r = rng(29)
+    L, D = 40, 64
+    q, k, v = (r.standard_normal((1, 1, L, D)).astype(np.float32) for _ in range(3))
+    got = O.flash_attention_v1(q, k, v)[0, 0]
+    q16, k16, v16 = (t.astype(np.float16).astype(np.float32)[0, 0] for t in (q, k, v))
+    for i in (0, 1, 17, 39):
+        s = np.array([np.float32(np.dot(q16[i].astype(np.float64), k16[j].astype(np.float64)))
+                      * np.float32(0.125) for j in range(i + 1)], dtype=np.float32)
+        p = np.exp(s - s.max()).astype(np.float32)
+        p16 = p.astype(np.float16).astype(np.float64)
+        out = (p16[:, None] * v16[:i + 1].astype(np.float64)).sum(0) / p.astype(np.float64).sum()
+        assert np.abs(got[i] - out).max() < 2e-6
+
+
+def test_attention_tile_size_only_moves_the_p_rounding():
+    r = rng(31)
+    q, k, v = (r.standard_normal((1, 2, 200, 64)).astype(np.float32) for _ in range(3))
+    a = O.flash_attention_v1(q, k, v, block=64)
+    b = O.flash_attention_v1(q, k, v, block=32)
+    assert 0 < np.abs(a - b).max() <= 2.0**-10 * np.abs(v).max()
+
+
+# ----------------------------------------------------------------------------- softmax
+def test_softmax_vs_torch():
+    r = rng(37)
+    x = (4 * r.standard_normal((33, 768))).astype(np.float32)
+    want = torch.softmax(torch.from_numpy(x).double(), -1).numpy()
+    got = O.softmax_rows(x)
+    assert np.abs(got - want).max() < 5e-7  # a few fp32 ulps of values <= 1
+    assert np.abs(got.sum(-1) - 1).max() < 1e-5
+    x16 = x.astype(np.float16)
+    got16 = O.softmax_rows(x16)
+    want16 = torch.softmax(torch.from_numpy(x16).double(), -1).numpy()
+    assert got16.dtype == np.float16
+    assert np.abs(got16.astype(np.float64) - want16).max() <= 2.0**-11
+
+
+# ----------------------------------------------------------------------------- whole model
+def gpt2_fp64(params, ids, n_head):
+    """An independently written GPT-2 (HF block order: ln_1 -> attn -> +res -> ln_2 -> mlp ->
+    +res -> ln_f) in fp64 torch, true-precision matmuls, library softmax/gelu/layer_norm."""
+    P = {k: torch.from_numpy(np.asarray(v)).double() for k, v in params.items()}
+    ids_t = torch.from_numpy(ids)
+    B, L = ids.shape
+    h = P["wte_weight"].shape[1]
+    d = h // n_head
+    F = torch.nn.functional
+    x = P["wte_weight"][ids_t] + P["wpe_weight"][:L]
+    mask = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    for i in range(O.n_layers_of(params)):
+        a, m = f"blocks.{i}.0.", f"blocks.{i}.1."
+        y = F.layer_norm(x, (h,), P[a + "layer_norm_weight"], P[a + "layer_norm_bias"], 1e-5)
+        qkv = y @ P[a + "c_attn_weight"] + P[a + "c_attn_bias"]
+        q, k, v = (t.view(B, L, n_head, d).permute(0, 2, 1, 3) for t in qkv.split(h, dim=-1))
+        s = (q @ k.transpose(-1, -2)) / math.sqrt(d)
+        s = s.masked_fill(~mask, float("-inf"))
+        o = (s.softmax(-1) @ v).permute(0, 2, 1, 3).reshape(B, L, h)
+        x = x + o @ P[a + "c_proj_weight"] + P[a + "c_proj_bias"]
+        y = F.layer_norm(x, (h,), P[m + "layer_norm_weight"], P[m + "layer_norm_bias"], 1e-5)
+        y = F.gelu(y @ P[m + "ffn1_weight"] + P[m + "ffn1_bias"], approximate="tanh")
+        x = x + y @ P[m + "ffn2_weight"] + P[m + "ffn2_bias"]
+    x = F.layer_norm(x, (h,), P["layer_norm_weight"], P["layer_norm_bias"], 1e-5)
+    return x.numpy(), (x @ P["wte_weight"].T).numpy()
+
+
+def test_model_composition_vs_independent_fp64_gpt2():
+    cfg = dict(n_layer=3, n_head=4, n_embd=128, vocab_size=211, block_size=96)
+    params = O.synthetic_params(**cfg, seed=7, std=0.08)
+    r = rng(41)
+    for k in params:  # non-trivial biases and LayerNorm affine so a dropped term shows
+        if k.endswith("_bias"):
+            params[k] = (0.05 * r.standard_normal(params[k].shape)).astype(np.float32)
+        elif "layer_norm_weight" in k:
+            params[k] = (1 + 0.1 * r.standard_normal(params[k].shape)).astype(np.float32)
+    ids = O.synthetic_ids(2, 80, cfg["vocab_size"], seed=7)
+    want_h, want_logits = gpt2_fp64(params, ids, cfg["n_head"])
+    got_h, got_logits = O.gpt2_forward(params, ids, cfg["n_head"], lm_head=True)
+    # fp16 operand rounding inside every product: ~1e-3 relative overall
+    assert np.abs(got_h - want_h).max() <= 5e-3 * np.abs(want_h).max()
+    assert np.abs(got_logits - want_logits).max() <= 5e-3 * np.abs(want_logits).max()
+    # and the bound discriminates: flipping the sign of one small (0.05 sigma) bias vector in
+    # the middle of the network already lands far outside it
+    bad = dict(params)
+    bad["blocks.1.1.ffn2_bias"] = -params["blocks.1.1.ffn2_bias"]
+    bad_h = O.gpt2_forward(bad, ids, cfg["n_head"])
+    assert np.abs(bad_h - want_h).max() > 2e-2 * np.abs(want_h).max()
