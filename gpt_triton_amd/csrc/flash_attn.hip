@@ -51,6 +51,13 @@ template <> struct Ld8<float> {
   }
 };
 
+// exp for the softmax: the fp32-storage build keeps the accurate library
+// routine (fewer fp16 rounding flips of P against the reference's np.exp);
+// the fp16-storage build uses the hardware exp2 path.
+template <typename T> __device__ __forceinline__ float softmax_exp(float x);
+template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float softmax_exp<_Float16>(float x) { return __expf(x); }
+
 __device__ __forceinline__ h8 zero_h8() {
   h8 z;
 #pragma unroll
@@ -100,50 +107,59 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
   if (last_q > L - 1) last_q = L - 1;
   const int nt = last_q / BKEY + 1;  // key tiles 0..nt-1 touch this query block
 
-  // ---- staging registers ---------------------------------------------------
-  h8 kreg[K_LD];            // waves 0-1
-  h8 vreg[V_UNITS][4];      // waves 2-3
+  // ---- staging: each thread moves NLD 16-byte chunks per tile --------------
+  // waves 0-1 (role K): chunk s = i*128 + st -> key s / CH, chunk s % CH
+  // waves 2-3 (role V): unit  s = (i/4)*128 + st -> key group s & 15 (4 keys),
+  //                     chunk s >> 4; register i holds key 4*group + i%4.
+  // Rows past the end of the sequence are clamped to the last row: their keys
+  // are masked (P = 0 exactly) and the values stay finite.
+  constexpr int NLD = K_LD;
+  static_assert(K_LD == 4 * V_UNITS, "K and V staging must move the same chunk count");
   const int st = tid & 127;
+  const bool role_k = wave < 2;
+  const T* sp = role_k ? Kp : Vp;
+  int srow[NLD], scol[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    if (role_k) {
+      const int s = i * 128 + st;
+      srow[i] = s / CH;
+      scol[i] = (s % CH) * 8;
+    } else {
+      const int s = (i >> 2) * 128 + st;
+      srow[i] = (s & 15) * 4 + (i & 3);
+      scol[i] = (s >> 4) * 8;
+    }
+  }
+  h8 stg[NLD];
 
   auto load_tile = [&](int t) {
     const int k0 = t * BKEY;
-    if (wave < 2) {
 #pragma unroll
-      for (int i = 0; i < K_LD; ++i) {
-        const int s = i * 128 + st, key = s / CH, c = s % CH;
-        kreg[i] = (k0 + key) < L ? Ld8<T>::load(Kp + (int64_t)(k0 + key) * D + c * 8)
-                                 : zero_h8();
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < V_UNITS; ++i) {
-        const int s = i * 128 + st, kg = s & 15, c = s >> 4;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const int key = k0 + kg * 4 + kk;
-          vreg[i][kk] = key < L ? Ld8<T>::load(Vp + (int64_t)key * D + c * 8) : zero_h8();
-        }
-      }
+    for (int i = 0; i < NLD; ++i) {
+      int row = k0 + srow[i];
+      row = row < L ? row : L - 1;
+      stg[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
     }
   };
 
   auto store_tile = [&](int stage) {
     char* ks_ = smem + stage * STAGE;
     char* vs_ = ks_ + K_BYTES;
-    if (wave < 2) {
+    if (role_k) {
 #pragma unroll
-      for (int i = 0; i < K_LD; ++i) {
-        const int s = i * 128 + st, key = s / CH, c = s % CH;
-        *reinterpret_cast<h8*>(ks_ + key * (D * 2) + ((c ^ (key & 7)) << 4)) = kreg[i];
+      for (int i = 0; i < NLD; ++i) {
+        const int key = srow[i], c = scol[i] >> 3;
+        *reinterpret_cast<h8*>(ks_ + key * (D * 2) + ((c ^ (key & 7)) << 4)) = stg[i];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < V_UNITS; ++i) {
-        const int s = i * 128 + st, kg = s & 15, c = s >> 4;
+      for (int u = 0; u < V_UNITS; ++u) {
+        const int kg = srow[4 * u] >> 2, d0 = scol[4 * u];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const int d = c * 8 + j;
-          h4 col = {vreg[i][0][j], vreg[i][1][j], vreg[i][2][j], vreg[i][3][j]};
+          const int d = d0 + j;
+          h4 col = {stg[4 * u][j], stg[4 * u + 1][j], stg[4 * u + 2][j], stg[4 * u + 3][j]};
           *reinterpret_cast<h4*>(vs_ + d * 128 + ((kg ^ ((d >> 1) & 15)) << 3)) = col;
         }
       }
@@ -198,13 +214,13 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
         }
       bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
       const float mnew = bmax > mrun ? bmax : mrun;
-      const float mult = __expf(mrun - mnew);
+      const float mult = softmax_exp<T>(mrun - mnew);
       float psum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float p = __expf(s[kb][r] - mnew);
+          const float p = softmax_exp<T>(s[kb][r] - mnew);
           s[kb][r] = p;
           psum += p;
         }
