@@ -9,27 +9,34 @@
 // here by the store instead of by three copies.
 //
 // Structure of one workgroup (WM x WN wavefronts):
-//   * a BM x BN output tile, K walked in steps of BK = 64 through a ring of
-//     STAGES LDS buffers filled by direct global->LDS loads (16 B per lane,
-//     no VGPR staging);
-//   * LDS rows are 128 B (64 halves) = 8 chunks of 16 B; chunk c of row r is
-//     kept at position c ^ (r & 7) so that the 16-byte fragment reads of 8
-//     consecutive rows hit 8 different bank groups;
+//   * a BM x BN output tile; K is walked in steps of BKS (32 or 64) through a
+//     ring of NST LDS stages filled by direct global->LDS loads (16 B per lane,
+//     no VGPR staging).  The ring is deep enough that the tile after the one
+//     being multiplied is already resident: the barrier that publishes tile
+//     kt+1 sits in front of the last k-step of tile kt, and the first fragments
+//     of tile kt+1 are read right behind it, so no MFMA waits for a barrier plus
+//     an LDS round trip;
+//   * LDS rows are BKS halves wide; the 16-byte chunks of a row are XOR-swizzled
+//     with a key taken from the row number so that the 16 lanes the LDS serves
+//     per clock (64 banks x 4 B) never share a bank:
+//         128-byte rows: chunk c of row r at c ^ ((r >> 1) & 7)
+//          64-byte rows: chunk c of row r at c ^ ((r >> 2) & 3)
 //   * each wavefront owns a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA blocks.
 //     The MFMA is issued as D[n][m] (weight rows as the first operand) so a
-//     lane ends up with 4 consecutive n for one m: an 8-byte packed store.
+//     lane ends up with 4 consecutive n for one m;
+//   * the epilogue applies bias/GELU in that layout, stages fp32 through LDS
+//     and stores row-major runs (see store_wave_tile);
 //   * workgroup ids are remapped so each XCD (ids are dealt round-robin over
 //     the 8 XCDs) gets a contiguous range of tiles, N fastest: the tiles that
 //     share a row block of A run on the same L2 at the same time.
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
 
 namespace gptmi {
 
 namespace {
-
-constexpr int BK = 64;
-constexpr int ROW_BYTES = BK * 2;  // 128
 
 struct EpiDev {
   const void* bias;
@@ -43,12 +50,22 @@ struct EpiDev {
   int d;
   int gelu;
   int vec_ok;  // pointers and N allow 4-element vector accesses
+#ifdef GPTMI_TUNING
+  unsigned long long* trace;  // tuning builds only: per-workgroup phase time stamps
+#endif
 };
 
-__device__ __forceinline__ void lds_dma16(const void* gsrc, void* ldst) {
-  __builtin_amdgcn_global_load_lds(
-      (const __attribute__((address_space(1))) void*)gsrc,
-      (__attribute__((address_space(3))) void*)ldst, 16, 0, 0);
+// Direct global->LDS load of 16 bytes per lane: lane l's bytes land at LDS
+// byte offset lds_off + 16*l (lds_off is wavefront-uniform and travels in M0).
+// Issued as inline assembly so that the compiler's wait-count tracking does not
+// see an LDS-writing memory instruction in flight: with the builtin, every LDS
+// wait inside the pipelined loop degrades to "wait for everything".  Completion
+// is tracked by hand with vmcnt (wait_vmcnt) ahead of the workgroup barrier.
+__device__ __forceinline__ void lds_dma16(const void* gsrc, unsigned lds_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_off), "v"(gsrc)
+               : "memory", "m0");
 }
 
 // Workgroup barrier that does not drain the vector-memory counter: the
@@ -60,158 +77,234 @@ __device__ __forceinline__ void block_barrier() {
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
-  if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  else if constexpr (N == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-  else if constexpr (N == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-  else if constexpr (N == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-  else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-  else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-  else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-  else if constexpr (N == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-  else static_assert(N < 0, "add this vmcnt value");
+  static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 template <typename T> struct Pack4;
 template <> struct Pack4<_Float16> { typedef h4 type; };
 template <> struct Pack4<float> { typedef f4 type; };
 
-// Applies bias/GELU/residual to 4 consecutive columns [n0, n0+4) of row m and
-// stores them.
+// Address of out[m][n] (plain) or of the q/k/v element that column n of row m
+// scatters to (qkv mode; n is a multiple of 4 and head sizes are too, so 4
+// consecutive columns stay inside one head).
 template <typename T, bool QKV>
-__device__ __forceinline__ void epilogue4(const EpiDev& ep, int64_t m, int n0, f4 acc,
-                                          int N) {
-  typedef typename Pack4<T>::type P;
-  const bool full = (n0 + 3 < N) && ep.vec_ok;
-  float z[4] = {acc[0], acc[1], acc[2], acc[3]};
-  if (ep.bias) {
-    const T* bp = (const T*)ep.bias + n0;
-    if (full) {
-      P b = *reinterpret_cast<const P*>(bp);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) z[j] += (float)b[j];
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n0 + j < N) z[j] += (float)bp[j];
-    }
-  }
-  if (ep.gelu) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) z[j] = gelu_new(z[j]);
-  }
+__device__ __forceinline__ T* out_ptr(const EpiDev& ep, int64_t m, int n, int N) {
   if constexpr (!QKV) {
-    const int64_t off = m * (int64_t)N + n0;
-    if (ep.residual) {
-      const T* rp = (const T*)ep.residual + off;
-      if (full) {
-        P r = __builtin_nontemporal_load(reinterpret_cast<const P*>(rp));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) z[j] += (float)r[j];
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (n0 + j < N) z[j] += (float)rp[j];
-      }
-    }
-    T* op = (T*)ep.out + off;
-    if (full) {
-      P o;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = (T)z[j];
-      *reinterpret_cast<P*>(op) = o;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n0 + j < N) op[j] = (T)z[j];
-    }
+    return (T*)ep.out + (m * (int64_t)N + n);
   } else {
-    // column n of the [q | k | v] matrix -> (which, head, dd); row m -> (b, l)
     const int hd = ep.heads * ep.d;
-    const int which = n0 / hd;
-    const int within = n0 - which * hd;
+    const int which = n / hd;
+    const int within = n - which * hd;
     const int head = within / ep.d;
     const int dd = within - head * ep.d;
     const int64_t b = m / ep.L;
     const int64_t l = m - b * ep.L;
     T* base = (T*)(which == 0 ? ep.q : (which == 1 ? ep.k : ep.v));
-    T* op = base + (((b * ep.heads + head) * ep.L + l) * ep.d + dd);
-    if (full) {
-      P o;
+    return base + (((b * ep.heads + head) * ep.L + l) * ep.d + dd);
+  }
+}
+
+constexpr int EP_STRIDE = 64 * 4 + 16;  // bytes of one staged epilogue row (64 fp32 + pad)
+constexpr int EP_SLAB = 32 * EP_STRIDE; // one wavefront's staging slab
+
+// Epilogue of one wavefront's (32*MB) x (32*NB) sub-tile whose first element is
+// (mw0, nw0).  A lane holds, per 32x32 block, m = lane%32 and for g = 0..3 the 4
+// columns 8g + 4*(lane/32) + 0..3.  Bias and GELU are applied in that layout,
+// the fp32 values are staged through the wavefront's private LDS slab (32 rows
+// x 64 columns, rows padded by 16 B) and read back row-major: 16 lanes cover one
+// row's 64 columns, so residual loads and output stores are contiguous 128-byte
+// (fp16) or 256-byte (fp32) runs per row.
+//   FAST: the workgroup tile lies entirely inside M x N and every pointer
+//   allows 4-element vector accesses -- straight-line code, no predicates.
+template <int MB, int NB, typename T, bool QKV, bool FAST, bool GELU, bool RES>
+__device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const EpiDev& ep,
+                                                  int64_t mw0, int nw0, int M, int N, char* slab,
+                                                  int lane) {
+  typedef typename Pack4<T>::type P4;
+  static_assert(NB % 2 == 0, "wave tile must be a multiple of 64 columns");
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int rrow = lane >> 4, rcol = (lane & 15) * 4;
+
+  // bias of this lane's columns, fetched once: [i][g] -> 4 consecutive columns
+  f4 bias_r[NB][4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = (T)z[j];
-      *reinterpret_cast<P*>(op) = o;
-    } else {
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n0 + j < N) op[j] = (T)z[j];
+    for (int g = 0; g < 4; ++g) {
+      const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
+      f4 b = {0.f, 0.f, 0.f, 0.f};
+      if (ep.bias) {
+        const T* bp = (const T*)ep.bias + n;
+        if (FAST) {
+          const P4 t = *reinterpret_cast<const P4*>(bp);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) b[e] = (float)bp[e];
+        }
+      }
+      bias_r[i][g] = b;
+    }
+
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+    const int64_t mbase = mw0 + j * 32;
+#pragma unroll
+    for (int i2 = 0; i2 < NB / 2; ++i2) {
+      const int n = nw0 + i2 * 64 + rcol;
+      // residual of the 8 row groups this lane stores, requested up front
+      P4 res[8];
+      if (RES && FAST) {
+#pragma unroll
+        for (int rr = 0; rr < 8; ++rr)
+          res[rr] = __builtin_nontemporal_load(reinterpret_cast<const P4*>(
+              (const T*)ep.residual + ((mbase + rr * 4 + rrow) * (int64_t)N + n)));
+      }
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int i = i2 * 2 + ii;
+          f4 z;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            z[e] = acc[i][j][4 * g + e] + bias_r[i][g][e];
+            if (GELU) z[e] = gelu_new(z[e]);
+          }
+          *reinterpret_cast<f4*>(slab + frow * EP_STRIDE + (ii * 32 + g * 8 + fhalf * 4) * 4) = z;
+        }
+      }
+#pragma unroll
+      for (int rr = 0; rr < 8; ++rr) {
+        const int row = rr * 4 + rrow;
+        const int64_t m = mbase + row;
+        f4 z = *reinterpret_cast<const f4*>(slab + row * EP_STRIDE + rcol * 4);
+        if (FAST) {
+          if (RES) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) z[e] += (float)res[rr][e];
+          }
+          P4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (T)z[e];
+#ifdef GPTMI_FAKE_STORE
+          *reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m & 255, n, N)) = o;
+#elif defined(GPTMI_PLAIN_STORE)
+          *reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m, n, N)) = o;
+#else
+          // streaming store: the output is not read again by this kernel and
+          // must not push the operand panels out of L2
+          __builtin_nontemporal_store(o, reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m, n, N)));
+#endif
+        } else {
+          if (m >= M || n >= N) continue;
+          T* op = out_ptr<T, QKV>(ep, m, n, N);
+          const T* rp = RES ? (const T*)ep.residual + (m * (int64_t)N + n) : nullptr;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) op[e] = (T)(z[e] + (RES ? (float)rp[e] : 0.f));
+        }
+      }
     }
   }
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, typename T, bool QKV>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(
-    const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N,
-    int Kp, int tiles_m, int tiles_n, EpiDev ep) {
+template <int MB, int NB, typename T, bool QKV>
+__device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDev& ep,
+                                                int64_t mw0, int nw0, int M, int N, bool fast,
+                                                char* slab, int lane) {
+  const bool res = !QKV && ep.residual != nullptr;
+#define GPTMI_EPI(F, G, R) \
+  store_wave_tile_v<MB, NB, T, QKV, F, G, R>(acc, ep, mw0, nw0, M, N, slab, lane)
+  if (fast) {
+    if (ep.gelu) { if (res) GPTMI_EPI(true, true, true); else GPTMI_EPI(true, true, false); }
+    else { if (res) GPTMI_EPI(true, false, true); else GPTMI_EPI(true, false, false); }
+  } else {
+    if (ep.gelu) { if (res) GPTMI_EPI(false, true, true); else GPTMI_EPI(false, true, false); }
+    else { if (res) GPTMI_EPI(false, false, true); else GPTMI_EPI(false, false, false); }
+  }
+#undef GPTMI_EPI
+}
+
+// XCD-aware tile id: workgroup ids are dealt round-robin over the 8 XCDs, so id
+// p runs on XCD p % 8.  The remap hands every XCD a contiguous range of tiles.
+__device__ __forceinline__ int xcd_tile(int pid, int num_tiles) {
+  const int per = (num_tiles + 7) >> 3;
+  int tall = num_tiles & 7;
+  if (tall == 0) tall = 8;
+  const int xcd = pid & 7, loc = pid >> 3;
+  return xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
+}
+
+// WPE = wavefronts per SIMD the register allocation must leave room for (two
+// 4-wavefront workgroups per CU need 2).
+template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
+__global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
+    const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
+    int tiles_m, int tiles_n, EpiDev ep) {
+  static_assert(BKS == 32 || BKS == 64, "k-step of 32 or 64");
+  static_assert(NST >= 3, "the pipeline keeps the next tile resident");
   constexpr int T_ = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int MB = TM / 32, NB = TN / 32;
-  constexpr int A_IT = BM * 8 / T_, B_IT = BN * 8 / T_;
-  constexpr int LPT = A_IT + B_IT;  // direct loads per thread per k-tile
-  constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
-  static_assert(BM * 8 % T_ == 0 && BN * 8 % T_ == 0, "tile/threads mismatch");
-  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
+  constexpr int ROWB = BKS * 2;            // bytes per LDS row
+  constexpr int CPR = ROWB / 16;           // 16-byte chunks per row (4 or 8)
+  constexpr int CSH = CPR == 8 ? 3 : 2;    // log2(CPR)
+  constexpr int KSH = CPR == 8 ? 1 : 2;    // swizzle key = (row >> KSH) & (CPR-1)
+  constexpr int A_IT = BM * CPR / T_, B_IT = BN * CPR / T_;
+  constexpr int LPT = A_IT + B_IT;         // direct loads per thread per k-tile
+  constexpr int STAGE = (BM + BN) * ROWB;
+  constexpr int KS = BKS / 16;             // MFMA k-steps per tile
+  static_assert(BM * CPR % T_ == 0 && BN * CPR % T_ == 0, "tile/threads mismatch");
+  static_assert(TM % 32 == 0 && TN % 64 == 0, "wave tile must be 32 x 64 aligned");
+  static_assert(NST * STAGE >= WM * WN * EP_SLAB, "epilogue staging does not fit");
+  static_assert((NST - 2) * LPT <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WM, wn = wave / WM;
-
-  // ---- XCD-aware tile id ------------------------------------------------
-  const int num_tiles = tiles_m * tiles_n;
-  int tile;
-  {
-    const int pid = blockIdx.x;
-    const int per = (num_tiles + 7) >> 3;
-    int tall = num_tiles & 7;
-    if (tall == 0) tall = 8;
-    const int xcd = pid & 7, loc = pid >> 3;
-    tile = xcd < tall ? xcd * per + loc
-                      : tall * per + (xcd - tall) * (per - 1) + loc;
-  }
+#ifdef GPTMI_TUNING
+  const unsigned long long t_start = __builtin_amdgcn_s_memtime();
+#endif
+  const int tile = xcd_tile(blockIdx.x, tiles_m * tiles_n);
   const int tn = tile % tiles_n, tm = tile / tiles_n;
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- per-thread sources of the direct global->LDS loads -----------------
-  // Linear 16-byte slot s of a tile: row s>>3, stored chunk position s&7,
-  // which holds source chunk (s&7) ^ (row&7).
-  const _Float16* a_src[A_IT];
-  const _Float16* b_src[B_IT];
+  // 16-byte slot s of an operand tile: row s / CPR, position s % CPR, which
+  // holds source chunk (s % CPR) ^ key(row).  Rows past the matrix edge re-read
+  // the last row (their products are never stored).
+  const char* a_src[A_IT];
+  const char* b_src[B_IT];
 #pragma unroll
   for (int it = 0; it < A_IT; ++it) {
-    const int s = it * T_ + tid, r = s >> 3, c = (s & 7) ^ (r & 7);
+    const int s = it * T_ + tid, r = s >> CSH, c = (s & (CPR - 1)) ^ ((r >> KSH) & (CPR - 1));
     int row = m0 + r;
     row = row < M ? row : M - 1;
-    a_src[it] = A + (size_t)row * Kp + c * 8;
+    a_src[it] = (const char*)(A + (size_t)row * Kp) + c * 16;
   }
 #pragma unroll
   for (int it = 0; it < B_IT; ++it) {
-    const int s = it * T_ + tid, r = s >> 3, c = (s & 7) ^ (r & 7);
+    const int s = it * T_ + tid, r = s >> CSH, c = (s & (CPR - 1)) ^ ((r >> KSH) & (CPR - 1));
     int row = n0 + r;
     row = row < N ? row : N - 1;
-    b_src[it] = Bt + (size_t)row * Kp + c * 8;
+    b_src[it] = (const char*)(Bt + (size_t)row * Kp) + c * 16;
   }
-
-  auto issue = [&](int stage, int kt) {
-    char* as = smem + stage * STAGE_BYTES;
-    char* bs = as + BM * ROW_BYTES;
+  const unsigned wave_off =
+      __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + (unsigned)wave * 1024u);
+  auto issue = [&](int kt) {
+    const unsigned as = wave_off + (kt % NST) * STAGE;
+    const unsigned bs = as + BM * ROWB;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it)
-      lds_dma16(a_src[it] + (size_t)kt * BK, as + (it * T_ + wave * 64) * 16);
+      lds_dma16(a_src[it] + (size_t)kt * ROWB, as + it * T_ * 16);
 #pragma unroll
     for (int it = 0; it < B_IT; ++it)
-      lds_dma16(b_src[it] + (size_t)kt * BK, bs + (it * T_ + wave * 64) * 16);
+      lds_dma16(b_src[it] + (size_t)kt * ROWB, bs + it * T_ * 16);
   };
 
   f16v acc[NB][MB];
@@ -222,67 +315,126 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int KT = Kp / BK;
+  // fragment read offsets (bytes) inside a stage
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> KSH) & (CPR - 1);
+  const int a_row_off = (wm * TM + frow) * ROWB;
+  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
+  h8 af[2][MB], bf[2][NB];
+  auto read_frags = [&](int kt, int ks, int slot) {
+    const char* st = smem + (kt % NST) * STAGE;
+    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
-    if (s < KT) issue(s, s);
-
-  // fragment read offsets (bytes) inside a stage: row-major 128-byte rows
-  const int frow = lane & 31, fhalf = lane >> 5, fsw = lane & 7;
-  const int a_row_off = (wm * TM + frow) * ROW_BYTES;
-  const int b_row_off = BM * ROW_BYTES + (wn * TN + frow) * ROW_BYTES;
-
-  for (int kt = 0; kt < KT; ++kt) {
-    // tile kt must have landed; up to STAGES-2 younger tiles may be in flight
-    if (kt + STAGES - 2 < KT) wait_vmcnt<(STAGES - 2) * LPT>();
-    else wait_vmcnt<0>();
-    block_barrier();
-    if (kt + STAGES - 1 < KT) issue((kt + STAGES - 1) % STAGES, kt + STAGES - 1);
-
-    const char* st = smem + (kt % STAGES) * STAGE_BYTES;
+    for (int j = 0; j < MB; ++j)
+      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      const int choff = ((ks * 2 + fhalf) ^ fsw) << 4;
-      h8 af[MB], bf[NB];
+    for (int i = 0; i < NB; ++i)
+      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
+  };
+  auto mma = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
       for (int j = 0; j < MB; ++j)
-        af[j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROW_BYTES + choff);
+        acc[i][j] =
+            __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j], 0, 0, 0);
+  };
+
+  const int KT = Kp / BKS;
+#ifdef GPTMI_NO_LOADS
+  constexpr bool loads = false;
+#else
+  constexpr bool loads = true;
+#endif
+  if (loads) {
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
-        bf[i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROW_BYTES + choff);
+    for (int s = 0; s < NST - 1; ++s)
+      if (s < KT) issue(s);
+    // tile 0 must have landed; up to NST-2 younger tiles stay in flight
+    if (KT >= NST - 1) wait_vmcnt<(NST - 2) * LPT>();
+    else wait_vmcnt<0>();
+  }
+  asm volatile("s_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+#ifdef GPTMI_TUNING
+  const unsigned long long t_pro = __builtin_amdgcn_s_memtime();
+#endif
+
+  // Fragments of the next k-step are requested before the MFMAs of this one
+  // issue; the scheduling fences keep the compiler from sinking the reads
+  // behind the MFMAs again.  In front of the last k-step of a tile the next
+  // tile is published (own loads landed, then the barrier) and the ring slot
+  // of tile kt-1, which every wavefront has finished reading, is refilled.
+  for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+    for (int ks = 0; ks < KS; ++ks) {
+      const int cur = ks & 1;
+      if (ks + 1 < KS) {
+        read_frags(kt, ks + 1, cur ^ 1);
+      } else {
+        if (kt + 1 < KT && loads) {
+          // tile kt+1 complete; tiles kt+2 .. kt+NST-2 may still be in flight
+          if (kt + NST - 2 < KT) wait_vmcnt<(NST - 3) * LPT>();
+          else wait_vmcnt<0>();
+        }
+        asm volatile("s_barrier" ::: "memory");
+        if (kt + NST - 1 < KT && loads) issue(kt + NST - 1);
+        read_frags(kt + 1, 0, cur ^ 1);  // past the last tile this reads a dead stage
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#ifndef GPTMI_NO_MFMA
+      mma(cur);
+#else
 #pragma unroll
-        for (int j = 0; j < MB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[i], af[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < MB; ++j) acc[0][j][0] += (float)af[cur][j][0] + (float)af[cur][j][7];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) acc[i][0][1] += (float)bf[cur][i][0] + (float)bf[cur][i][7];
+#endif
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
-  // ---- epilogue: lane holds, per block, m = lane%32 and for g = 0..3 the 4
-  // columns 8g + 4*(lane/32) + 0..3 -----------------------------------------
+  // ---- epilogue -----------------------------------------------------------
+#ifdef GPTMI_TUNING
+  const unsigned long long t_loop = __builtin_amdgcn_s_memtime();
+#endif
+#ifdef GPTMI_NO_EPILOGUE
+  {
+    float keep = 0.f;  // consumes every accumulator so that no MFMA is dead code
 #pragma unroll
-  for (int j = 0; j < MB; ++j) {
-    const int64_t m = (int64_t)m0 + wm * TM + j * 32 + frow;
-    if (m >= M) continue;
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
+      for (int j = 0; j < MB; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * TN + i * 32 + g * 8 + fhalf * 4;
-        if (n >= N) continue;
-        f4 v4 = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                 acc[i][j][4 * g + 3]};
-        epilogue4<T, QKV>(ep, m, n, v4, N);
-      }
-    }
+        for (int r = 0; r < 16; ++r) keep += acc[i][j][r];
+    if (keep == 123.456f) ((T*)ep.out)[tid] = (T)keep;
   }
+#else
+  block_barrier();  // every wavefront is done reading the operand stages
+  const bool fast = ep.vec_ok && n0 + BN <= N && m0 + BM <= M;
+  store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM, n0 + wn * TN, M, N, fast,
+                                  smem + wave * EP_SLAB, lane);
+#endif
+#ifdef GPTMI_TUNING
+  if (ep.trace && tid == 0) {
+    unsigned hw, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    unsigned long long* t = ep.trace + (size_t)blockIdx.x * 6;
+    t[0] = t_start;
+    t[1] = t_pro;
+    t[2] = t_loop;
+    t[3] = __builtin_amdgcn_s_memtime();
+    t[4] = hw;
+    t[5] = xcc;
+  }
+#endif
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, typename T, bool QKV>
-int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp,
-               const EpiDev& ep, hipStream_t st) {
-  auto kern = gemm_kernel<BM, BN, WM, WN, STAGES, T, QKV>;
-  constexpr int smem = STAGES * (BM + BN) * ROW_BYTES;
+template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
+int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+               hipStream_t st) {
+  auto kern = gemm_kernel<BM, BN, WM, WN, BKS, NST, WPE, T, QKV>;
+  constexpr int smem = NST * (BM + BN) * BKS * 2;
   static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -294,31 +446,36 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp,
     attr_done = true;
   }
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (N + BN - 1) / BN;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(WM * WN * 64), smem,
-                     st, (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m,
-                     tiles_n, ep);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(WM * WN * 64), smem, st,
+                     (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n,
+                     ep);
   return 0;
 }
 
 template <typename T, bool QKV>
-int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp,
-                 const EpiDev& ep, hipStream_t st) {
-  // Big problems: 256x256 tiles, 8 waves.  Small ones: 128x128, 4 waves, so
-  // that tests with a few hundred rows still spread over several CUs.
+int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+                 hipStream_t st) {
+  // Big problems: 256x256 tiles, 8 wavefronts.  Small ones: 128x128, 4
+  // wavefronts, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256)
-    return launch_cfg<256, 256, 2, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
-  return launch_cfg<128, 128, 2, 2, 3, T, QKV>(A, Bt, M, N, Kp, ep, st);
+    return launch_cfg<256, 256, 2, 4, 32, 5, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 
 }  // namespace
 
-int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
-                const GemmEpilogue& e, hipStream_t st) {
+#ifndef GPTMI_TUNING
+int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const GemmEpilogue& e,
+                hipStream_t st) {
   if (M >= (1ll << 31) - 512) {
     set_error("gemm: M=%lld does not fit the kernel's 32-bit row index", (long long)M);
     return -2;
   }
-  EpiDev ep;
+  if (e.qkv && (e.d % 4) != 0) {
+    set_error("gemm qkv epilogue: head size %d must be a multiple of 4", e.d);
+    return -2;
+  }
+  EpiDev ep = {};
   ep.bias = e.bias;
   ep.residual = e.residual;
   ep.out = e.out;
@@ -330,21 +487,16 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
   ep.d = e.d;
   ep.gelu = e.gelu;
   const uintptr_t amask = e.f16 ? 7 : 15;
-  bool vec = (N % 4) == 0;
   auto aligned = [&](const void* p) { return p == nullptr || ((uintptr_t)p & amask) == 0; };
-  vec = vec && aligned(e.bias) && aligned(e.residual) && aligned(e.out) && aligned(e.q) &&
-        aligned(e.k) && aligned(e.v);
-  if (e.qkv) vec = vec && (e.d % 4) == 0;
+  const bool vec = (N % 4) == 0 && aligned(e.bias) && aligned(e.residual) && aligned(e.out) &&
+                   aligned(e.q) && aligned(e.k) && aligned(e.v);
   ep.vec_ok = vec ? 1 : 0;
-  if (e.qkv && (e.d % 4) != 0) {
-    set_error("gemm qkv epilogue: head size %d must be a multiple of 4", e.d);
-    return -2;
-  }
   if (e.f16)
     return e.qkv ? launch_shape<_Float16, true>(A, Bt, M, N, Kp, ep, st)
                  : launch_shape<_Float16, false>(A, Bt, M, N, Kp, ep, st);
   return e.qkv ? launch_shape<float, true>(A, Bt, M, N, Kp, ep, st)
                : launch_shape<float, false>(A, Bt, M, N, Kp, ep, st);
 }
+#endif
 
 }  // namespace gptmi
