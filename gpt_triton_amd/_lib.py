@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libgptmi.so")
 
 GPTMI_F32, GPTMI_F16 = 0, 1
-GPTMI_W_KN, GPTMI_W_NK = 0, 1
+GPTMI_W_KN, GPTMI_W_NK, GPTMI_W_PACKED = 0, 1, 2
 GPTMI_O_BNLD, GPTMI_O_BLND = 0, 1
 
 _vp, _i64, _int, _f32, _u64, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
@@ -22,10 +22,12 @@ SIGNATURES = {
     "gptmi_layernorm": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _int, _vp]),
     "gptmi_softmax": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "gptmi_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),
+    "gptmi_packed_weight_bytes": (_sz, [_i64, _i64]),
+    "gptmi_pack_weight": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp]),
     "gptmi_linear": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _f32, _u64, _int,
                             _vp, _sz, _int, _vp]),
-    "gptmi_linear_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp,
-                                _sz, _int, _vp]),
+    "gptmi_linear_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                                _vp, _sz, _int, _vp]),
     "gptmi_flash_attn": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _f32,
                                 _u64, _int, _int, _vp]),
 }

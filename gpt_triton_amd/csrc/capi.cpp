@@ -44,7 +44,8 @@ static LinearPlan plan_linear(int64_t M, int64_t N, int64_t K, int dtype, int wl
   LinearPlan p;
   p.Kp = (int)round_up(K, 64);
   p.pack_x = !(dtype == GPTMI_F16 && p.Kp == K);
-  const bool pack_w = !(wlayout == GPTMI_W_NK && dtype == GPTMI_F16 && p.Kp == K);
+  const bool pack_w = !(wlayout == GPTMI_W_PACKED ||
+                        (wlayout == GPTMI_W_NK && dtype == GPTMI_F16 && p.Kp == K));
   p.w_off = 0;
   p.w_bytes = pack_w ? (size_t)round_up(N * (int64_t)p.Kp * 2, 256) : 0;
   p.x_off = p.w_bytes;
@@ -158,13 +159,37 @@ size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, 
   return plan_linear(M, N, K, dtype, wlayout).total;
 }
 
+size_t gptmi_packed_weight_bytes(int64_t N, int64_t K) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)round_up(N * round_up(K, 64) * 2, 256);
+}
+
+int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wlayout, int dtype,
+                      void* stream) {
+  if (!W || !packed || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
+      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK) || N > (1 << 30) || K > (1 << 30)) {
+    set_error("pack_weight: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (((uintptr_t)packed & 255) != 0) {
+    set_error("pack_weight: destination must be 256-byte aligned");
+    return GPTMI_ERR_INVALID;
+  }
+  const int Kp = (int)round_up(K, 64);
+  if (wlayout == GPTMI_W_KN)
+    launch_pack_transpose(W, packed, (int)K, (int)N, Kp, dtype == GPTMI_F16, (hipStream_t)stream);
+  else
+    launch_pack_rows(W, packed, N, (int)K, Kp, dtype == GPTMI_F16, (hipStream_t)stream);
+  return check_launch("pack_weight");
+}
+
 int gptmi_linear(const void* x, const void* W, const void* bias, const void* residual,
                  void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
                  uint64_t seed, int wlayout, void* workspace, size_t workspace_bytes,
                  int dtype, void* stream) {
   (void)seed;
   if (!x || !W || !out || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
-      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK)) {
+      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK && wlayout != GPTMI_W_PACKED)) {
     set_error("linear: invalid argument");
     return GPTMI_ERR_INVALID;
   }
@@ -200,9 +225,10 @@ int gptmi_linear(const void* x, const void* W, const void* bias, const void* res
 
 int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, void* k,
                      void* v, int64_t B, int64_t L, int64_t heads, int64_t d, int64_t K,
-                     void* workspace, size_t workspace_bytes, int dtype, void* stream) {
+                     int wlayout, void* workspace, size_t workspace_bytes, int dtype,
+                     void* stream) {
   if (!x || !W || !q || !k || !v || B <= 0 || L <= 0 || heads <= 0 || d <= 0 || K <= 0 ||
-      !dtype_ok(dtype)) {
+      !dtype_ok(dtype) || (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_PACKED)) {
     set_error("linear_qkv: invalid argument");
     return GPTMI_ERR_INVALID;
   }
@@ -218,8 +244,8 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, vo
   hipStream_t st = (hipStream_t)stream;
   const void *A, *Bt;
   int Kp;
-  int rc = prepare_operands(x, W, M, N, K, dtype, GPTMI_W_KN, workspace, workspace_bytes, st,
-                            &A, &Bt, &Kp);
+  int rc = prepare_operands(x, W, M, N, K, dtype, wlayout, workspace, workspace_bytes, st, &A,
+                            &Bt, &Kp);
   if (rc) return rc;
   if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) {
     set_error("linear_qkv: x and W must be 16-byte aligned");

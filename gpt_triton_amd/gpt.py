@@ -15,13 +15,14 @@ Differences, all additive: GPU_TO_FLOPS knows "mi355x"; FusedGPT.forward takes
 `FusedGPT.forward` reads `config.dropout` (the reference reads a `dropout_prob` attribute the
 dataclass does not have, gpt.py:165, and so only works in eval mode).
 """
+import re
 from dataclasses import dataclass
 
 import torch
 import torch.nn as nn
 
 from .kernels import (flash_attention_v1, fused_embeddings, fused_ffn, fused_layer_norm, lm_head,
-                      matmul_and_split_qkv)
+                      matmul_and_split_qkv, pack_weight)
 
 # dense fp16/bf16 tensor throughput, FLOP/s
 GPU_TO_FLOPS = {
@@ -30,6 +31,27 @@ GPU_TO_FLOPS = {
     "h100": 989 * 10**12,
     "mi355x": 2500 * 10**12,
 }
+
+
+class _PackedWeights:
+    """Per-module cache of the GEMM's packed weight images, used in eval mode only.  An entry
+    is rebuilt when the parameter's storage, dtype or version counter changes (optimizer steps,
+    load_state_dict, .to()); in-place edits made through `param.data` bypass the version
+    counter -- call `clear()` (or `model.train()`) after those."""
+
+    def __init__(self):
+        self._entries = {}
+
+    def get(self, name, param):
+        key = (param.data_ptr(), param._version, param.dtype, tuple(param.shape))
+        hit = self._entries.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, pack_weight(param.data))
+            self._entries[name] = hit
+        return hit[1]
+
+    def clear(self):
+        self._entries.clear()
 
 
 def _linear_flops(tokens, fan_in, fan_out):
@@ -56,18 +78,29 @@ class FusedAttention(nn.Module):
         self.c_attn_bias = nn.Parameter(torch.rand(3 * h))
         self.c_proj_weight = nn.Parameter(torch.rand(h, h))
         self.c_proj_bias = nn.Parameter(torch.rand(h))
+        self._packed = _PackedWeights()
+
+    def _weight(self, name):
+        prm = getattr(self, name)
+        if self.training or (self.hidden_size // self.num_heads) % 8 != 0:
+            return prm.data
+        return self._packed.get(name, prm)
+
+    def train(self, mode=True):
+        self._packed.clear()
+        return super().train(mode)
 
     def forward(self, x):
         p = self.dropout_prob if self.training else 0.0
         skip = x
         y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
-        q, k, v = matmul_and_split_qkv(y, self.c_attn_weight.data, self.c_attn_bias.data,
+        q, k, v = matmul_and_split_qkv(y, self._weight("c_attn_weight"), self.c_attn_bias.data,
                                        self.num_heads)
         # [B, N, L, d] values in a [B, L, N, d] buffer: the head merge below copies nothing
         y = flash_attention_v1(q, k, v, dropout_prob=p, merged_heads_layout=True)
         y = y.transpose(1, 2).contiguous().view(skip.shape)
-        return fused_ffn(y, self.c_proj_weight.data, bias=self.c_proj_bias.data, residual=skip,
-                         add_gelu=False, dropout_prob=p)
+        return fused_ffn(y, self._weight("c_proj_weight"), bias=self.c_proj_bias.data,
+                         residual=skip, add_gelu=False, dropout_prob=p)
 
     def get_fwd_flops(self, num_tokens):
         h = self.hidden_size
@@ -90,14 +123,23 @@ class FusedMLP(nn.Module):
         self.ffn1_bias = nn.Parameter(torch.rand(mid))
         self.ffn2_weight = nn.Parameter(torch.rand(mid, h))
         self.ffn2_bias = nn.Parameter(torch.rand(h))
+        self._packed = _PackedWeights()
+
+    def _weight(self, name):
+        prm = getattr(self, name)
+        return prm.data if self.training else self._packed.get(name, prm)
+
+    def train(self, mode=True):
+        self._packed.clear()
+        return super().train(mode)
 
     def forward(self, x):
         p = self.dropout_prob if self.training else 0.0
         skip = x
         y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
-        y = fused_ffn(y, self.ffn1_weight.data, bias=self.ffn1_bias.data, residual=None,
+        y = fused_ffn(y, self._weight("ffn1_weight"), bias=self.ffn1_bias.data, residual=None,
                       add_gelu=True, dropout_prob=p)
-        return fused_ffn(y, self.ffn2_weight.data, bias=self.ffn2_bias.data, residual=skip,
+        return fused_ffn(y, self._weight("ffn2_weight"), bias=self.ffn2_bias.data, residual=skip,
                          add_gelu=False, dropout_prob=p)
 
     def get_fwd_flops(self, num_tokens):
@@ -167,6 +209,9 @@ class FusedGPT(nn.Module):
         return self
 
 
+_MASK_BUFFER = re.compile(r"h\.\d+\.attn\.(bias|masked_bias)")  # HF's causal-mask buffers
+
+
 def convert_huggingface_to_triton(hf_sd, hf_config):
     """Renames a HuggingFace GPT2Model state dict to FusedGPT's keys.  HF's Conv1D weights are
     already [in, out], so no tensor is transposed; the causal-mask buffers are dropped."""
@@ -189,7 +234,7 @@ def convert_huggingface_to_triton(hf_sd, hf_config):
             rename[f"h.{i}.{src}"] = f"blocks.{i}.{dst}"
     sd = {}
     for key, tensor in hf_sd.items():
-        if key.endswith("attn.bias") or key.endswith("attn.masked_bias"):
+        if _MASK_BUFFER.fullmatch(key):
             continue
         sd[rename[key]] = tensor
     return sd, config

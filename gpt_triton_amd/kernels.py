@@ -9,9 +9,11 @@ pointers to one entry point of libgptmi.so (include/gptmi.h).
     matmul_and_split_qkv(x, weight, bias, num_heads)             kernels.py:347-367
     flash_attention_v1(q, k, v, dropout_prob=0.0)                kernels.py:477-525
 
-plus `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:318-342) and
+plus `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:318-342),
 `lm_head(x, wte)` (the transposed-weight product the reference leaves as a TODO,
-gpt.py:159-161).  Tensors must live on the GPU: there is no CPU path.  dropout_prob > 0
+gpt.py:159-161) and `pack_weight(weight)`: the GEMM reads its weight as an fp16,
+K-contiguous image which `fused_ffn` / `matmul_and_split_qkv` otherwise rebuild on every
+call; a `PackedWeight` may be passed wherever they take `weight`.  Tensors must live on the GPU: there is no CPU path.  dropout_prob > 0
 raises NotImplementedError.
 """
 import math
@@ -53,6 +55,42 @@ def _workspace(nbytes, device):
     if nbytes == 0:
         return None
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+class PackedWeight:
+    """The fp16 [N][round_up(K, 64)] image of a [K, N] weight (see gptmi_pack_weight).  `shape`
+    and `dtype` are those of the weight it was made from, so it can stand in for it."""
+
+    __slots__ = ("data", "shape", "dtype", "device")
+
+    def __init__(self, data, shape, dtype):
+        self.data, self.shape, self.dtype, self.device = data, tuple(shape), dtype, data.device
+
+    def is_contiguous(self):
+        return True
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+@torch.no_grad()
+def pack_weight(weight):
+    """Packs a contiguous [K, N] weight once; the result replaces `weight` in `fused_ffn` and
+    `matmul_and_split_qkv` and must be rebuilt when the weight changes."""
+    assert weight.dim() == 2 and weight.is_contiguous()
+    dev = _on_gpu(weight)
+    K_, N = weight.shape
+    lib = _lib.load()
+    buf = torch.empty(lib.gptmi_packed_weight_bytes(N, K_), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_pack_weight(weight.data_ptr(), buf.data_ptr(), N, K_, _lib.GPTMI_W_KN,
+                                   _dtype_code(weight, "pack_weight"), _stream())
+    _lib.check(rc, "pack_weight")
+    return PackedWeight(buf, weight.shape, weight.dtype)
+
+
+def _wlayout(weight, default):
+    return _lib.GPTMI_W_PACKED if isinstance(weight, PackedWeight) else default
 
 
 @torch.no_grad()
@@ -157,7 +195,8 @@ def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False, dropout_prob=
         residual = residual.view(z.shape)
         assert residual.is_contiguous()
 
-    _linear(x, weight, bias, residual, z, add_gelu, dropout_prob, _lib.GPTMI_W_KN, "fused_ffn")
+    _linear(x, weight, bias, residual, z, add_gelu, dropout_prob,
+            _wlayout(weight, _lib.GPTMI_W_KN), "fused_ffn")
     return z.view((*out_shape_0, N))
 
 
@@ -195,6 +234,8 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
     code = _dtype_code(x, "matmul_and_split_qkv")
     if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         raise TypeError("matmul_and_split_qkv: x, weight and bias must share a dtype")
+    if head_size % 8 != 0 and isinstance(weight, PackedWeight):
+        raise NotImplementedError("matmul_and_split_qkv: packed weights need head_size % 8 == 0")
     if head_size % 8 != 0:
         # the scatter epilogue stores 8-element groups; other head sizes take the plain GEMM
         y = fused_ffn(x, weight, bias=bias)
@@ -207,12 +248,13 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
     v = torch.empty(shape, device=dev, dtype=x.dtype)
     lib = _lib.load()
     M, K, N = batch_size * seqlen, x.shape[2], 3 * hidden_size
-    ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, _lib.GPTMI_W_KN)
+    wl = _wlayout(weight, _lib.GPTMI_W_KN)
+    ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, wl)
     ws = _workspace(ws_bytes, dev)
     with torch.cuda.device(dev):
         rc = lib.gptmi_linear_qkv(x.data_ptr(), weight.data_ptr(), _ptr(bias), q.data_ptr(),
                                   k.data_ptr(), v.data_ptr(), batch_size, seqlen, num_heads,
-                                  head_size, K, _ptr(ws), ws_bytes, code, _stream())
+                                  head_size, K, wl, _ptr(ws), ws_bytes, code, _stream())
     _lib.check(rc, "matmul_and_split_qkv")
     return q, k, v
 

@@ -47,7 +47,8 @@ typedef enum gptmi_status {
 /* Layout of the weight operand of gptmi_linear. */
 typedef enum gptmi_wlayout {
   GPTMI_W_KN = 0, /* W[K][N] row-major: the reference's (and HF Conv1D's) in x out layout */
-  GPTMI_W_NK = 1  /* W[N][K] row-major: out x in, e.g. the tied LM head over wte[V][H] */
+  GPTMI_W_NK = 1, /* W[N][K] row-major: out x in, e.g. the tied LM head over wte[V][H] */
+  GPTMI_W_PACKED = 2 /* the fp16 [N][round_up(K,64)] image written by gptmi_pack_weight */
 } gptmi_wlayout;
 
 /* Layout of the output of gptmi_flash_attn. */
@@ -107,6 +108,23 @@ size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype,
                                     int wlayout);
 
 /*
+ * Bytes of the packed image of a [K][N] weight: fp16 [N][round_up(K, 64)].
+ */
+size_t gptmi_packed_weight_bytes(int64_t N, int64_t K);
+
+/*
+ * Writes the packed image of W (layout GPTMI_W_KN or GPTMI_W_NK, storage `dtype`)
+ * into `packed` (gptmi_packed_weight_bytes(N, K) bytes, 256-byte aligned): the
+ * weight rounded to fp16, K-contiguous, zero padded to a multiple of 64.  It is
+ * what gptmi_linear builds in its workspace on every call; packing once and
+ * passing GPTMI_W_PACKED skips that step for weights that do not change.
+ * No counterpart in the reference (its Triton kernel reads W[K][N] in place,
+ * kernels.py:231-234).
+ */
+int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wlayout,
+                      int dtype, void* stream);
+
+/*
  * out = gelu?(x @ W + bias) + residual
  * Operands of the product are rounded to fp16, products and sums are fp32
  * (MFMA), then in fp32: + bias, tanh-GELU if `gelu`, + residual; one rounding
@@ -114,7 +132,8 @@ size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype,
  *
  * Replaces fused_ffn(x, weight, bias, residual, add_gelu, dropout_prob) ->
  * kernels.py:260-315 and fused_ffn_kernel -> kernels.py:169-257.
- *   x [M][K]   W [K][N] (GPTMI_W_KN) or [N][K] (GPTMI_W_NK)   bias [N] or NULL
+ *   x [M][K]   W [K][N] (GPTMI_W_KN), [N][K] (GPTMI_W_NK) or packed (GPTMI_W_PACKED)
+ *   bias [N] or NULL
  *   residual [M][N] or NULL     out [M][N]
  * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
  * (may be NULL when that is 0).  p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
@@ -132,13 +151,13 @@ int gptmi_linear(const void* x, const void* W, const void* bias,
  *
  * Replaces matmul_and_split_qkv(x, weight, bias, num_heads) -> kernels.py:347-367
  * (fused_ffn followed by split + 3 x view/transpose/contiguous copies).
- *   x [B*L][K]   W [K][3*heads*d] (GPTMI_W_KN)   bias [3*heads*d] or NULL
+ *   x [B*L][K]   W [K][3*heads*d] (GPTMI_W_KN) or packed   bias [3*heads*d] or NULL
  *   q, k, v [B][heads][L][d]       d a multiple of 8
  */
 int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
                      void* k, void* v, int64_t B, int64_t L, int64_t heads,
-                     int64_t d, int64_t K, void* workspace, size_t workspace_bytes,
-                     int dtype, void* stream);
+                     int64_t d, int64_t K, int wlayout, void* workspace,
+                     size_t workspace_bytes, int dtype, void* stream);
 
 /*
  * out = softmax(causal(q k^T * scale)) v, mask "key index <= query index".
