@@ -44,6 +44,11 @@ def load():
         raise RuntimeError(
             f"{LIB_PATH} is missing: build the HIP extension first "
             "(`python -m gpt_triton_amd.build`, needs hipcc); there is no CPU fallback")
+    # PyTorch ships its own HIP runtime; it must be in the process before libgptmi.so is, so
+    # that the library binds to that copy (the one whose streams and allocations it is handed)
+    # instead of pulling in a second runtime from /opt/rocm.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
