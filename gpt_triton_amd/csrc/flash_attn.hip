@@ -286,9 +286,265 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Resident-K/V variant for short sequences (L*D small enough that K and V^T of
+// one (batch, head) fit in half a CU's LDS, e.g. L <= 320 at D = 64).
+//
+// One workgroup = 4 wavefronts = one (batch, head).  K ([L][D], 16-byte chunks
+// swizzled with (row >> 1) & 7) and V^T ([D][Lp + 4], Lp = L rounded up to 64;
+// the 8 pad bytes per row spread the 32 rows a fragment read touches over all
+// banks) are staged once, behind ONE barrier; after it the wavefronts never
+// synchronise again.  Queries are cut into chunks of 32; chunk c costs
+// c/2 + 1 key tiles (causal), and the chunks are dealt to the 4 wavefronts in
+// snake order from the most expensive one, which balances the triangle (L = 300:
+// 8, 8, 7, 7 tiles).  The arithmetic per tile is that of the tiled kernel.
+// ---------------------------------------------------------------------------
+template <int D, typename T, bool BLND>
+__global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
+    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+    T* __restrict__ O, int heads, int L, float scale) {
+  constexpr int CH = D / 8, KS = D / 16, DB = D / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int Lp = (L + BKEY - 1) / BKEY * BKEY;
+  const int vstride = 2 * Lp + 8;            // bytes per V^T row
+  char* ks_ = smem;                          // K: L rows of D halves
+  char* vs_ = smem + (size_t)L * D * 2;      // V^T: D rows of Lp (+4) halves
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.x;
+  const int64_t base = (int64_t)bh * L * D;
+  const T* Qp = Q + base;
+  const T* Kp = K + base;
+  const T* Vp = V + base;
+
+  // ---- stage K: chunk s -> row s / CH, chunk s % CH --------------------------
+  for (int s0 = 0; s0 < L * CH; s0 += 256 * 4) {
+    h8 r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int s = s0 + i * 256 + tid;
+      if (s < L * CH) r[i] = Ld8<T>::load(Kp + (int64_t)(s / CH) * D + (s % CH) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int s = s0 + i * 256 + tid;
+      if (s < L * CH) {
+        const int row = s / CH, c = s % CH;
+        *reinterpret_cast<h8*>(ks_ + row * (D * 2) + ((c ^ ((row >> 1) & 7)) << 4)) = r[i];
+      }
+    }
+  }
+  // ---- stage V^T: unit u -> d-chunk u % CH, key group u / CH (4 keys) ---------
+  // keys past the end repeat the last row: their weights are exactly 0
+  const int units = (Lp / 4) * CH;
+  for (int u0 = 0; u0 < units; u0 += 256) {
+    const int u = u0 + tid;
+    if (u < units) {
+      const int c = u % CH, kg = u / CH;
+      h8 r[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        int key = kg * 4 + kk;
+        key = key < L ? key : L - 1;
+        r[kk] = Ld8<T>::load(Vp + (int64_t)key * D + c * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        h4 col = {r[0][j], r[1][j], r[2][j], r[3][j]};
+        *reinterpret_cast<h4*>(vs_ + (c * 8 + j) * vstride + kg * 8) = col;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int ql = lane & 31, g = lane >> 5;
+  const int nc = (L + 31) / 32;
+  // snake deal: position i (chunk nc-1-i) goes to wavefront i%8 < 4 ? i%8 : 7 - i%8
+  for (int i0 = 0; i0 < nc; i0 += 8) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int i = i0 + (half == 0 ? wave : 7 - wave);
+      if (i >= nc) continue;
+      const int qw0 = (nc - 1 - i) * 32;  // first query of the chunk
+      const int q = qw0 + ql;
+      h8 qf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        qf[ks] = q < L ? Ld8<T>::load(Qp + (int64_t)q * D + ks * 16 + g * 8) : zero_h8();
+      f16v oacc[DB];
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[b][r] = 0.f;
+      float mrun = -INFINITY, den = 0.f;
+      int last_q = qw0 + 31;
+      if (last_q > L - 1) last_q = L - 1;
+      const int nt = last_q / BKEY + 1;
+      for (int t = 0; t < nt; ++t) {
+        const int k0 = t * BKEY;
+        // ---- S^T = K . Q^T -----------------------------------------------------
+        f16v s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+          int key = k0 + kb * 32 + ql;
+          key = key < L ? key : L - 1;  // masked anyway; keeps the read inside K
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const h8 kf = *reinterpret_cast<const h8*>(
+                ks_ + key * (D * 2) + (((ks * 2 + g) ^ ((key >> 1) & 7)) << 4));
+            s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+          }
+        }
+        // ---- causal mask, running max, exponentials -----------------------------
+        const bool need_mask = k0 + BKEY - 1 > qw0;
+        if (need_mask) {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+              s[kb][r] = key <= q ? s[kb][r] : -INFINITY;
+            }
+        }
+        float mult, psum = 0.f;
+        if constexpr (sizeof(T) == 2) {
+          // fp16 storage: the running max is kept on the raw scores and scale * log2(e) is
+          // folded into one fused multiply-add in front of exp2 -- the same real-number
+          // formula as the reference, two VALU operations per score fewer
+          const float c = scale * 1.4426950408889634f;
+          float bmax = -INFINITY;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, s[kb][r]);
+          bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+          const float mnew = bmax > mrun ? bmax : mrun;
+          mult = __builtin_amdgcn_exp2f((mrun - mnew) * c);
+          const float m2 = mnew * c;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][r], c, -m2));
+              s[kb][r] = p;
+              psum += p;
+            }
+          mrun = mnew;
+        } else {
+          // fp32 storage: the reference's operation order, library exp
+          float bmax = -INFINITY;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              s[kb][r] *= scale;
+              bmax = fmaxf(bmax, s[kb][r]);
+            }
+          bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+          const float mnew = bmax > mrun ? bmax : mrun;
+          mult = softmax_exp<T>(mrun - mnew);
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float p = softmax_exp<T>(s[kb][r] - mnew);
+              s[kb][r] = p;
+              psum += p;
+            }
+          mrun = mnew;
+        }
+        psum += __shfl_xor(psum, 32, kWave);
+        den = den * mult + psum;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[b][r] *= mult;
+        // ---- O^T += V^T . P^T --------------------------------------------------
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt) {
+            h8 pf;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pf[j] = (_Float16)s[kb][8 * tt + j];
+            const int kbase = k0 + kb * 32 + tt * 16 + 4 * g;  // first of this lane's keys
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+              const char* row = vs_ + (b * 32 + ql) * vstride + kbase * 2;
+              const h4 lo = *reinterpret_cast<const h4*>(row);
+              const h4 hi = *reinterpret_cast<const h4*>(row + 16);
+              h8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+              oacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[b], 0, 0, 0);
+            }
+          }
+      }
+      // ---- out[q][d] = O^T[d][q] / den ------------------------------------------
+      if (q < L) {
+        int64_t row_off;
+        if (BLND) {
+          const int b = bh / heads, n = bh - b * heads;
+          row_off = (((int64_t)b * L + q) * heads + n) * D;
+        } else {
+          row_off = base + (int64_t)q * D;
+        }
+        const float inv = __builtin_amdgcn_rcpf(den);  // fp16 storage only (1 ulp of fp32)
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const int d = b * 32 + 8 * rg + 4 * g;
+            if constexpr (sizeof(T) == 2) {
+              h4 o;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) o[j] = (_Float16)(oacc[b][4 * rg + j] * inv);
+              *reinterpret_cast<h4*>(O + row_off + d) = o;
+            } else {
+              f4 o;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) o[j] = oacc[b][4 * rg + j] / den;
+              *reinterpret_cast<f4*>(O + row_off + d) = o;
+            }
+          }
+      }
+    }
+  }
+}
+
+// LDS bytes of the resident variant, or 0 if this (L, D) does not fit two workgroups per CU.
+inline size_t resident_lds_bytes(int L, int D) {
+  const int Lp = (L + BKEY - 1) / BKEY * BKEY;
+  const size_t bytes = (size_t)L * D * 2 + (size_t)D * (2 * Lp + 8);
+  return bytes <= 80 * 1024 ? bytes : 0;
+}
+
+template <int D, typename T, bool BLND>
+int launch_resident(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                    int L, float scale, size_t lds, hipStream_t st) {
+  auto kern = flash_attn_resident_kernel<D, T, BLND>;
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(80 KB LDS): %s", hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)BN), dim3(256), lds, st, (const T*)q, (const T*)k,
+                     (const T*)v, (T*)out, heads, L, scale);
+  return 0;
+}
+
 template <int D, typename T>
 int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
              int heads, int L, float scale, bool blnd, hipStream_t st) {
+  if (const size_t lds = resident_lds_bytes(L, D)) {
+    return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
+                : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
+  }
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
   if (blnd)
     hipLaunchKernelGGL((flash_attn_kernel<D, T, true>), grid, dim3(256), 0, st,
