@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
   constexpr int STAGE = 2 * K_BYTES;
   constexpr int K_LD = BKEY * CH / 128; // K chunks per staging thread
   constexpr int V_UNITS = 16 * CH / 128; // (4 keys x 8 d) units per staging thread
-  __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // 2 * STAGE bytes
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.x;
@@ -546,12 +546,28 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
                 : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
   }
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
+  constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V^T tile
+  auto k_blnd = flash_attn_kernel<D, T, true>;
+  auto k_bnld = flash_attn_kernel<D, T, false>;
+  static bool attr_done = false;  // idempotent; a race only repeats the calls
+  if (!attr_done && lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_blnd),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_bnld),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", lds, hipGetErrorString(e));
+      return -4;
+    }
+  }
+  attr_done = true;
   if (blnd)
-    hipLaunchKernelGGL((flash_attn_kernel<D, T, true>), grid, dim3(256), 0, st,
-                       (const T*)q, (const T*)k, (const T*)v, (T*)out, heads, L, scale);
+    hipLaunchKernelGGL(k_blnd, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
+                       (T*)out, heads, L, scale);
   else
-    hipLaunchKernelGGL((flash_attn_kernel<D, T, false>), grid, dim3(256), 0, st,
-                       (const T*)q, (const T*)k, (const T*)v, (T*)out, heads, L, scale);
+    hipLaunchKernelGGL(k_bnld, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
+                       (T*)out, heads, L, scale);
   return 0;
 }
 
@@ -561,8 +577,9 @@ int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
   switch (d) {
     case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
     case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
+    case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
     default:
-      set_error("flash_attn: head size %d not built (64 and 128 are)", d);
+      set_error("flash_attn: head size %d not built (64, 128 and 256 are)", d);
       return -2;
   }
 }

@@ -452,309 +452,13 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
   return 0;
 }
 
-// ---------------------------------------------------------------------------
-// Persistent variant for large problems: one workgroup per CU walks a list of
-// tiles (virtual id = blockIdx + round * gridDim, mapped like the id of a
-// one-tile workgroup).  The LDS ring keeps running across tile boundaries --
-// the first k-tiles of the next output tile are already in flight while the
-// epilogue of the current one executes -- which removes the per-tile pipeline
-// fill and the idle time between the end of one workgroup and the start of the
-// next.  The epilogue stages through 32 KB of LDS outside the ring, one 32x32
-// fp32 block (4 KB) per wavefront at a time, 16-byte units XOR-swizzled with
-// (row >> 1) & 7.
-// ---------------------------------------------------------------------------
-constexpr int PS_SLAB = 32 * 32 * 4;  // one wavefront's 32x32 fp32 staging block
-
-template <int MB, int NB, typename T, bool QKV, bool FAST, bool GELU, bool RES>
-__device__ __forceinline__ void store_wave_tile_ps(f16v (&acc)[NB][MB], const EpiDev& ep,
-                                                   int64_t mw0, int nw0, int M, int N, char* slab,
-                                                   int lane) {
-  typedef typename Pack4<T>::type P4;
-  const int frow = lane & 31, fhalf = lane >> 5;
-  const int rrow = lane >> 3, runit = lane & 7;  // read back: 8 lanes per 32-column row
-#pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    // bias of this lane's columns of block column i
-    f4 bias_r[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
-      f4 b = {0.f, 0.f, 0.f, 0.f};
-      if (ep.bias) {
-        const T* bp = (const T*)ep.bias + n;
-        if (FAST) {
-          const P4 t = *reinterpret_cast<const P4*>(bp);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n + e < N) b[e] = (float)bp[e];
-        }
-      }
-      bias_r[g] = b;
-    }
-    const int n = nw0 + i * 32 + runit * 4;
-#pragma unroll
-    for (int j = 0; j < MB; ++j) {
-      const int64_t mbase = mw0 + j * 32;
-      P4 res[4];
-      if (RES && FAST) {
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr)
-          res[rr] = __builtin_nontemporal_load(reinterpret_cast<const P4*>(
-              (const T*)ep.residual + ((mbase + rr * 8 + rrow) * (int64_t)N + n)));
-      }
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f4 z;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          z[e] = acc[i][j][4 * g + e] + bias_r[g][e];
-          if (GELU) z[e] = gelu_new(z[e]);
-        }
-        const int unit = (g * 2 + fhalf) ^ ((frow >> 1) & 7);
-        *reinterpret_cast<f4*>(slab + frow * 128 + unit * 16) = z;
-      }
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int row = rr * 8 + rrow;
-        const int64_t m = mbase + row;
-        f4 z = *reinterpret_cast<const f4*>(slab + row * 128 + ((runit ^ ((row >> 1) & 7)) << 4));
-        if (FAST) {
-          if (RES) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) z[e] += (float)res[rr][e];
-          }
-          P4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (T)z[e];
-          __builtin_nontemporal_store(o, reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m, n, N)));
-        } else {
-          if (m >= M || n >= N) continue;
-          T* op = out_ptr<T, QKV>(ep, m, n, N);
-          const T* rp = RES ? (const T*)ep.residual + (m * (int64_t)N + n) : nullptr;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n + e < N) op[e] = (T)(z[e] + (RES ? (float)rp[e] : 0.f));
-        }
-      }
-    }
-  }
-}
-
-template <int BM, int BN, int WM, int WN, int NST, typename T, bool QKV>
-__global__ __launch_bounds__(WM * WN * 64, 2) void gemm_persistent_kernel(
-    const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
-    int tiles_m, int tiles_n, EpiDev ep) {
-  constexpr int BKS = 32, ROWB = 64, CPR = 4;
-  constexpr int T_ = WM * WN * 64;
-  constexpr int TM = BM / WM, TN = BN / WN;
-  constexpr int MB = TM / 32, NB = TN / 32;
-  constexpr int A_IT = BM * CPR / T_, B_IT = BN * CPR / T_;
-  constexpr int LPT = A_IT + B_IT;
-  constexpr int STAGE = (BM + BN) * ROWB;
-  static_assert(NST >= 3 && (NST - 2) * LPT <= 63, "ring depth");
-  static_assert(BM * CPR % T_ == 0 && BN * CPR % T_ == 0, "tile/threads mismatch");
-
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  char* slab = smem + NST * STAGE + (threadIdx.x >> 6) * PS_SLAB;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave % WM, wn = wave / WM;
-  const int num_tiles = tiles_m * tiles_n;
-  const int KT = Kp / BKS;  // >= NST - 1, checked by the launcher
-
-  // sources of the direct loads of one tile: slot s -> row s/4, chunk (s%4) ^ ((row>>2)&3).
-  // Only the (clamped) global row numbers depend on the tile; they are kept for the current
-  // and the next tile, the addresses are formed when a load is issued.
-  int a_cur[A_IT], b_cur[B_IT], a_nxt[A_IT], b_nxt[B_IT];
-  int a_coff[A_IT], b_coff[B_IT];
-#pragma unroll
-  for (int it = 0; it < A_IT; ++it) {
-    const int s = it * T_ + tid, r = s >> 2;
-    a_coff[it] = ((s & 3) ^ ((r >> 2) & 3)) * 16;
-  }
-#pragma unroll
-  for (int it = 0; it < B_IT; ++it) {
-    const int s = it * T_ + tid, r = s >> 2;
-    b_coff[it] = ((s & 3) ^ ((r >> 2) & 3)) * 16;
-  }
-  auto sources = [&](int tile, int (&a)[A_IT], int (&b)[B_IT]) {
-    const int tn = tile % tiles_n, tm = tile / tiles_n;
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      const int row = tm * BM + ((it * T_ + tid) >> 2);
-      a[it] = row < M ? row : M - 1;
-    }
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it) {
-      const int row = tn * BN + ((it * T_ + tid) >> 2);
-      b[it] = row < N ? row : N - 1;
-    }
-  };
-  const unsigned wave_off =
-      __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + (unsigned)wave * 1024u);
-  // g = running k-step count over all tiles of this workgroup (ring slot g % NST)
-  auto issue = [&](int g, const int (&a)[A_IT], const int (&b)[B_IT], int kt) {
-    const unsigned as = wave_off + (g % NST) * STAGE;
-    const unsigned bs = as + BM * ROWB;
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it)
-      lds_dma16((const char*)(A + (size_t)a[it] * Kp) + a_coff[it] + (size_t)kt * ROWB,
-                as + it * T_ * 16);
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it)
-      lds_dma16((const char*)(Bt + (size_t)b[it] * Kp) + b_coff[it] + (size_t)kt * ROWB,
-                bs + it * T_ * 16);
-  };
-
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 2) & 3;
-  const int a_row_off = (wm * TM + frow) * ROWB;
-  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
-  h8 af[2][MB], bf[2][NB];
-  auto read_frags = [&](int g, int ks, int slot) {
-    const char* st = smem + (g % NST) * STAGE;
-    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
-#pragma unroll
-    for (int j = 0; j < MB; ++j)
-      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
-  };
-
-  int vpid = blockIdx.x;
-  int tile = xcd_tile(vpid, num_tiles);
-  sources(tile, a_cur, b_cur);
-#pragma unroll
-  for (int s = 0; s < NST - 1; ++s) issue(s, a_cur, b_cur, s);
-  wait_vmcnt<(NST - 2) * LPT>();
-  asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
-
-  int g = 0;  // ring position of the current tile's k-tile 0
-  while (true) {
-    const int next_vpid = vpid + gridDim.x;
-    const bool has_next = next_vpid < num_tiles;
-    if (has_next) sources(xcd_tile(next_vpid, num_tiles), a_nxt, b_nxt);
-
-    f16v acc[NB][MB];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int j = 0; j < MB; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    for (int kt = 0; kt < KT; ++kt) {
-      // ---- k-step 0 of this k-tile: fragments were requested one step earlier
-      read_frags(g + kt, 1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[0][i], af[0][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      // ---- publish k-tile kt+1, refill the slot of k-tile kt-1, k-step 1
-      const bool more = kt + 1 < KT || has_next;
-      if (more) {
-        // loads in flight beyond k-tile kt+1: NST-3 tiles unless the stream is ending
-        if (kt + NST - 2 < KT || has_next) wait_vmcnt<(NST - 3) * LPT>();
-        else wait_vmcnt<0>();
-      }
-      asm volatile("s_barrier" ::: "memory");
-      {
-        const int kk = kt + NST - 1;
-        if (kk < KT) issue(g + kk, a_cur, b_cur, kk);
-        else if (has_next) issue(g + kk, a_nxt, b_nxt, kk - KT);
-      }
-      read_frags(g + kt + 1, 0, 0);  // at the very end this reads a dead slot
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-
-    // ---- epilogue of this tile; the next tile's first k-tiles are in flight
-    {
-      const int tn = tile % tiles_n, tm = tile / tiles_n;
-      const int m0 = tm * BM, n0 = tn * BN;
-      const bool fast = ep.vec_ok && n0 + BN <= N && m0 + BM <= M;
-      const bool res = !QKV && ep.residual != nullptr;
-      const int64_t mw0 = (int64_t)m0 + wm * TM;
-      const int nw0 = n0 + wn * TN;
-#define GPTMI_EPI(F, G, R) \
-  store_wave_tile_ps<MB, NB, T, QKV, F, G, R>(acc, ep, mw0, nw0, M, N, slab, lane)
-      if (fast) {
-        if (ep.gelu) { if (res) GPTMI_EPI(true, true, true); else GPTMI_EPI(true, true, false); }
-        else { if (res) GPTMI_EPI(true, false, true); else GPTMI_EPI(true, false, false); }
-      } else {
-        if (ep.gelu) { if (res) GPTMI_EPI(false, true, true); else GPTMI_EPI(false, true, false); }
-        else { if (res) GPTMI_EPI(false, false, true); else GPTMI_EPI(false, false, false); }
-      }
-#undef GPTMI_EPI
-    }
-    if (!has_next) break;
-    g += KT;
-    vpid = next_vpid;
-    tile = xcd_tile(vpid, num_tiles);
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it) a_cur[it] = a_nxt[it];
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it) b_cur[it] = b_nxt[it];
-  }
-}
-
-template <int BM, int BN, int WM, int WN, int NST, typename T, bool QKV>
-int launch_persistent(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
-                      hipStream_t st) {
-  auto kern = gemm_persistent_kernel<BM, BN, WM, WN, NST, T, QKV>;
-  constexpr int smem = NST * (BM + BN) * 64 + WM * WN * PS_SLAB;
-  static int num_cus = 0;  // idempotent one-time setup; a race only repeats it
-  if (num_cus == 0) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
-      return -4;
-    }
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        cus <= 0) {
-      set_error("cannot query the CU count");
-      return -4;
-    }
-    num_cus = cus;
-  }
-  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (N + BN - 1) / BN;
-  const int num_tiles = tiles_m * tiles_n;
-  // a multiple of 8 workgroups keeps the id -> XCD relation of the tile remap
-  int grid = num_cus - num_cus % 8;
-  if (grid > num_tiles) grid = num_tiles;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), smem, st,
-                     (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n, ep);
-  return 0;
-}
-
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
-  // Big problems: 256x256 tiles, 8 wavefronts; the persistent variant when there are
-  // enough tiles that the ragged last round over the CUs costs little (ffn1, qkv at the
-  // GPT-2 sizes), one workgroup per tile otherwise.  Small problems: 128x128 tiles, 4
-  // wavefronts, so that a few hundred rows still spread over several CUs.
-  if (M >= 2048 && N >= 256) {
-    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (tiles >= 4096 && Kp >= 32 * 4)
-      return launch_persistent<256, 256, 4, 2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  // Big problems: 256x256 tiles, 8 wavefronts, 5-stage ring (all 160 KB of LDS).  Small ones:
+  // 128x128 tiles, 4 wavefronts, so that a few hundred rows still spread over several CUs.
+  if (M >= 2048 && N >= 256)
     return launch_cfg<256, 256, 2, 4, 32, 5, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
-  }
   return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 

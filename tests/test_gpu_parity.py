@@ -201,6 +201,19 @@ def test_fused_ffn_gpt2_shapes(K, gpu_device, dtype, M, N, Kd, gelu, use_res):
     check(host(z), O.fused_ffn(x, w, bias=b, residual=res, add_gelu=gelu), dtype, "ffn")
 
 
+def test_fused_ffn_xl_shapes(K, gpu_device):
+    """BASELINE config 4 widths (d_model 1600, 25 heads, FFN 6400): N = 4800 / 1600 / 6400 are
+    not multiples of the 256-wide tile, K = 1600 / 6400 are multiples of 32 only."""
+    for (M, N, Kd, gelu, use_res) in [(2304, 4800, 1600, False, False), (2304, 6400, 1600, True, False),
+                                      (2304, 1600, 6400, False, True)]:
+        x, w, b, res = ffn_inputs(M, N, Kd, torch.float16, seed=N, gaussian=True)
+        res = res if use_res else None
+        z = K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device),
+                        residual=None if res is None else dev(res, gpu_device), add_gelu=gelu)
+        check(host(z), O.fused_ffn(x, w, bias=b, residual=res, add_gelu=gelu), torch.float16,
+              f"xl ffn {M}x{N}x{Kd}")
+
+
 def test_fused_ffn_leading_dims_and_residual_view(K, gpu_device):
     x, w, b, res = ffn_inputs(6 * 50, 128, 128, torch.float32, seed=9, gaussian=True)
     z = K.fused_ffn(dev(x.reshape(6, 50, 128), gpu_device), dev(w, gpu_device),
@@ -246,12 +259,26 @@ def attn_inputs(B, N, L, D, dtype, gaussian, seed=1337):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("B,N", [(3, 9), (2, 7)])
 @pytest.mark.parametrize("L", [199, 128, 63])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 def test_flash_attention_reference_grid(K, gpu_device, dtype, B, N, L, D):
     q, k, v = attn_inputs(B, N, L, D, dtype, gaussian=False)
     z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
     assert z.shape == (B, N, L, D) and z.dtype == dtype and z.is_contiguous()
     check_attention(host(z), O.flash_attention_v1(q, k, v), v, dtype, "attention")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_flash_attention_reference_golden_vectors(K, gpu_device, dtype):
+    """Against outputs of the reference's own kernel (Triton CPU interpreter), committed under
+    tests/golden/ -- not against the oracle."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "flash_attention_v1.npz"))
+    for n in "abc":
+        q, k, v = (z[f"{n}_{t}"].astype(NP[dtype]) for t in "qkv")
+        want = z[f"{n}_out"]
+        got = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+        check_attention(host(got), want, v, dtype, f"golden {n}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
@@ -274,6 +301,14 @@ def test_flash_attention_merged_heads_layout(K, gpu_device, dtype):
     assert b.shape == a.shape
     assert b.transpose(1, 2).is_contiguous()  # the model's head merge is then a no-op
     assert torch.equal(a, b)
+
+
+def test_flash_attention_xl_sequence(K, gpu_device):
+    """BASELINE config 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
+    K/V do not fit the resident variant)."""
+    q, k, v = attn_inputs(1, 5, 1024, 64, torch.float16, gaussian=True, seed=11)
+    z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+    check(host(z), O.flash_attention_v1(q, k, v), torch.float16, "attention L=1024")
 
 
 def test_flash_attention_is_causal(K, gpu_device):

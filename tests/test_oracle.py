@@ -257,6 +257,28 @@ def test_attention_tile_size_only_moves_the_p_rounding():
     assert 0 < np.abs(a - b).max() <= 2.0**-10 * np.abs(v).max()
 
 
+def test_attention_vs_reference_golden_vectors():
+    """tests/golden/flash_attention_v1.npz holds outputs of the reference's own
+    flash_attention_v1 (Triton CPU interpreter, tests/golden/make_flash_vectors.py).  They pin
+    what no closed form does: the fp16 rounding of P relative to the per-tile running max.  The
+    oracle reproduces them to the last bit except for fp32 summation order inside matmul."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "flash_attention_v1.npz"))
+    for n in "abc":
+        q, k, v = (z[f"{n}_{t}"].astype(np.float32) for t in "qkv")
+        want = z[f"{n}_out"]
+        got = O.flash_attention_v1(q, k, v)
+        diff = np.abs(got.astype(np.float64) - want)
+        assert diff.max() <= 2e-7 * np.abs(want).max()
+        assert (diff == 0).mean() > 0.95
+        # and the vectors themselves are sane: within the P-rounding distance of the textbook
+        assert np.abs(want - attention_fp64(q, k, v)).max() <= 2.0**-11 * np.abs(v).max()
+        # a tile of 32 instead of 64 moves the rounding and is told apart by the vectors
+        other = O.flash_attention_v1(q, k, v, block=32)
+        assert np.abs(other.astype(np.float64) - want).max() > 20 * diff.max()
+
+
 # ----------------------------------------------------------------------------- softmax
 def test_softmax_vs_torch():
     r = rng(37)
