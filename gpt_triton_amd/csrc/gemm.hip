@@ -11,11 +11,11 @@
 // Structure of one workgroup (WM x WN wavefronts):
 //   * a BM x BN output tile; K is walked in steps of BKS (32 or 64) through a
 //     ring of NST LDS stages filled by direct global->LDS loads (16 B per lane,
-//     no VGPR staging).  The ring is deep enough that the tile after the one
-//     being multiplied is already resident: the barrier that publishes tile
-//     kt+1 sits in front of the last k-step of tile kt, and the first fragments
-//     of tile kt+1 are read right behind it, so no MFMA waits for a barrier plus
-//     an LDS round trip;
+//     no VGPR staging).  NST >= 3: the tile after the one being multiplied is
+//     already resident -- the barrier that publishes tile kt+1 sits in front of
+//     the last k-step of tile kt and the first fragments of tile kt+1 are read
+//     right behind it, so no MFMA waits for a barrier plus an LDS round trip.
+//     NST == 2: plain double buffering (all a 256x256x64 stage leaves room for);
 //   * LDS rows are BKS halves wide; the 16-byte chunks of a row are XOR-swizzled
 //     with a key taken from the row number so that the 16 lanes the LDS serves
 //     per clock (64 banks x 4 B) never share a bank:
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
     int tiles_m, int tiles_n, EpiDev ep) {
   static_assert(BKS == 32 || BKS == 64, "k-step of 32 or 64");
-  static_assert(NST >= 3, "the pipeline keeps the next tile resident");
+  static_assert(NST >= 2, "at least double buffering");
   constexpr int T_ = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int MB = TM / 32, NB = TN / 32;
@@ -354,11 +354,38 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     else wait_vmcnt<0>();
   }
   asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
+  if constexpr (NST > 2) read_frags(0, 0, 0);
 #ifdef GPTMI_TUNING
   const unsigned long long t_pro = __builtin_amdgcn_s_memtime();
 #endif
 
+  if constexpr (NST == 2) {
+    // Plain double buffering (the only depth a 256x256x64 stage leaves room for): tile kt+1
+    // streams in while tile kt is multiplied; one barrier per tile.
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt > 0) {
+        if (loads) wait_vmcnt<0>();
+        block_barrier();
+      }
+      if (kt + 1 < KT && loads) issue(kt + 1);
+      read_frags(kt, 0, 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int cur = ks & 1;
+        if (ks + 1 < KS) read_frags(kt, ks + 1, cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef GPTMI_NO_MFMA
+        mma(cur);
+#else
+#pragma unroll
+        for (int j = 0; j < MB; ++j) acc[0][j][0] += (float)af[cur][j][0] + (float)af[cur][j][7];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) acc[i][0][1] += (float)bf[cur][i][0] + (float)bf[cur][i][7];
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else {
   // Fragments of the next k-step are requested before the MFMAs of this one
   // issue; the scheduling fences keep the compiler from sinking the reads
   // behind the MFMAs again.  In front of the last k-step of a tile the next
@@ -373,7 +400,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       } else {
         if (kt + 1 < KT && loads) {
           // tile kt+1 complete; tiles kt+2 .. kt+NST-2 may still be in flight
-          if (kt + NST - 2 < KT) wait_vmcnt<(NST - 3) * LPT>();
+          if (kt + NST - 2 < KT) wait_vmcnt<(NST > 2 ? (NST - 3) * LPT : 0)>();
           else wait_vmcnt<0>();
         }
         asm volatile("s_barrier" ::: "memory");
@@ -391,6 +418,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #endif
       __builtin_amdgcn_sched_barrier(0);
     }
+  }
   }
 
   // ---- epilogue -----------------------------------------------------------
@@ -455,10 +483,12 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
-  // Big problems: 256x256 tiles, 8 wavefronts, 5-stage ring (all 160 KB of LDS).  Small ones:
-  // 128x128 tiles, 4 wavefronts, so that a few hundred rows still spread over several CUs.
+  // Big problems: 256x256 tiles, 8 wavefronts (4x2, wave tile 64x128), K step 64 -- full
+  // 128-byte rows per direct load move ~1.5x the bytes per clock of 64-byte rows -- double
+  // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
+  // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256)
-    return launch_cfg<256, 256, 2, 4, 32, 5, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+    return launch_cfg<256, 256, 4, 2, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 
