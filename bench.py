@@ -68,6 +68,25 @@ def cpu_baseline(sample_batch=16, reps=2):
                       f"mean of {reps} after 1 warm-up, {dt * 1e3:.0f} ms per forward"}
 
 
+def copy_calibration(dev, rows=262144, cols=2048, reps=3):
+    """pack_rows_kernel on an fp16 [rows][cols] matrix whose width is already a multiple of 64
+    is an element-for-element copy: rows*cols*2 bytes read, the same written."""
+    import torch
+
+    from gpt_triton_amd import _lib
+
+    lib = _lib.load()
+    src = torch.randn(rows, cols, device=dev, dtype=torch.float16)
+    dst = torch.empty(lib.gptmi_packed_weight_bytes(rows, cols), dtype=torch.uint8, device=dev)
+    assert dst.numel() == src.numel() * 2
+    for _ in range(reps):
+        _lib.check(lib.gptmi_pack_weight(src.data_ptr(), dst.data_ptr(), rows, cols,
+                                         _lib.GPTMI_W_NK, _lib.GPTMI_F16,
+                                         torch.cuda.current_stream().cuda_stream), "copy calibration")
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.float16).view(rows, cols), src)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,6 +94,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the host-CPU leg (used under rocprofv3)")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also launch a plain copy kernel of known size (1 GiB read, 1 GiB "
+                         "written) so that FETCH_SIZE / WRITE_SIZE counters of the same "
+                         "rocprofv3 --pmc run can be scaled to bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's full share of the forward; "
@@ -162,6 +185,8 @@ def main():
                      "traffic": FFN1_TRAFFIC_BYTES},
     }
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
+    if args.traffic_calibration:
+        copy_calibration(dev)
     print(json.dumps(line), flush=True)
 
 

@@ -93,16 +93,30 @@ __device__ __forceinline__ T* out_ptr(const EpiDev& ep, int64_t m, int n, int N)
   if constexpr (!QKV) {
     return (T*)ep.out + (m * (int64_t)N + n);
   } else {
-    const int hd = ep.heads * ep.d;
-    const int which = n / hd;
-    const int within = n - which * hd;
-    const int head = within / ep.d;
-    const int dd = within - head * ep.d;
-    const int64_t b = m / ep.L;
-    const int64_t l = m - b * ep.L;
+    // m < 2^31 (checked by the launcher) and L <= m's range: 32-bit divisions
+    const unsigned hd = (unsigned)(ep.heads * ep.d);
+    const unsigned which = (unsigned)n / hd;
+    const unsigned within = (unsigned)n - which * hd;
+    const unsigned head = within / (unsigned)ep.d;
+    const unsigned dd = within - head * (unsigned)ep.d;
+    const unsigned L = (unsigned)ep.L;
+    const unsigned b = (unsigned)m / L;
+    const unsigned l = (unsigned)m - b * L;
     T* base = (T*)(which == 0 ? ep.q : (which == 1 ? ep.k : ep.v));
-    return base + (((b * ep.heads + head) * ep.L + l) * ep.d + dd);
+    return base + ((((int64_t)b * ep.heads + head) * ep.L + l) * ep.d + dd);
   }
+}
+
+// Head-major destination of column n, row 0 of batch 0: q/k/v base + (head * L + 0) * d + dd.
+template <typename T>
+__device__ __forceinline__ T* qkv_column_base(const EpiDev& ep, int n) {
+  const unsigned hd = (unsigned)(ep.heads * ep.d);
+  const unsigned which = (unsigned)n / hd;
+  const unsigned within = (unsigned)n - which * hd;
+  const unsigned head = within / (unsigned)ep.d;
+  const unsigned dd = within - head * (unsigned)ep.d;
+  T* base = (T*)(which == 0 ? ep.q : (which == 1 ? ep.k : ep.v));
+  return base + ((int64_t)head * ep.L * ep.d + dd);
 }
 
 constexpr int EP_STRIDE = 64 * 4 + 16;  // bytes of one staged epilogue row (64 fp32 + pad)
@@ -148,6 +162,22 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
       }
       bias_r[i][g] = b;
     }
+
+  // head-major scatter: the column part of the address once per 64-column slab, the row part
+  // (b, l) = divmod(m, L) once for the lane's first row and then by stepping -- the sub-tile
+  // spans fewer than 256 rows, so it crosses at most one batch boundary when L >= 256
+  T* qkv_col[NB / 2];
+  unsigned b0 = 0, l0 = 0;
+  const unsigned Lu = (unsigned)ep.L;
+  const bool step_rows = Lu >= 32u * MB;
+  if (QKV && FAST) {
+#pragma unroll
+    for (int i2 = 0; i2 < NB / 2; ++i2) qkv_col[i2] = qkv_column_base<T>(ep, nw0 + i2 * 64 + rcol);
+    const unsigned m_first = (unsigned)mw0 + (unsigned)rrow;
+    b0 = m_first / Lu;
+    l0 = m_first - b0 * Lu;
+  }
+  const int64_t batch_stride = (int64_t)ep.heads * ep.L * ep.d;
 
 #pragma unroll
   for (int j = 0; j < MB; ++j) {
@@ -197,7 +227,22 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
 #else
           // streaming store: the output is not read again by this kernel and
           // must not push the operand panels out of L2
-          __builtin_nontemporal_store(o, reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m, n, N)));
+          T* dst;
+          if constexpr (QKV) {
+            unsigned b, l;
+            if (step_rows) {
+              b = b0;
+              l = l0 + (unsigned)(j * 32 + rr * 4);
+              if (l >= Lu) { l -= Lu; ++b; }
+            } else {
+              b = (unsigned)m / Lu;
+              l = (unsigned)m - b * Lu;
+            }
+            dst = qkv_col[i2] + ((int64_t)b * batch_stride + (int64_t)l * ep.d);
+          } else {
+            dst = out_ptr<T, QKV>(ep, m, n, N);
+          }
+          __builtin_nontemporal_store(o, reinterpret_cast<P4*>(dst));
 #endif
         } else {
           if (m >= M || n >= N) continue;
@@ -244,7 +289,7 @@ __device__ __forceinline__ int xcd_tile(int pid, int num_tiles) {
 template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
 __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
-    int tiles_m, int tiles_n, EpiDev ep) {
+    int tiles_m, int tiles_n, int group_w, EpiDev ep) {
   static_assert(BKS == 32 || BKS == 64, "k-step of 32 or 64");
   static_assert(NST >= 2, "at least double buffering");
   constexpr int T_ = WM * WN * 64;
@@ -270,8 +315,14 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #ifdef GPTMI_TUNING
   const unsigned long long t_start = __builtin_amdgcn_s_memtime();
 #endif
+  // Tile order: the column tiles are cut into groups of group_w; inside a group the column
+  // runs fastest, then the row block, and the groups follow each other.  Workgroups that run
+  // at the same time then share few weight panels, which stay in the XCD's L2.
   const int tile = xcd_tile(blockIdx.x, tiles_m * tiles_n);
-  const int tn = tile % tiles_n, tm = tile / tiles_n;
+  const int grp = tile / (tiles_m * group_w);
+  const int in_grp = tile - grp * tiles_m * group_w;
+  const int grp_w = min(group_w, tiles_n - grp * group_w);
+  const int tm = in_grp / grp_w, tn = grp * group_w + in_grp % grp_w;
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- per-thread sources of the direct global->LDS loads -----------------
@@ -458,6 +509,23 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #endif
 }
 
+#ifdef GPTMI_TUNING
+int g_group_w = 0;
+#endif
+
+// Width, in column tiles, of the groups the tile order walks through.  The weight panels of
+// one group (group_w * BN rows of Kp halves) should stay in a 4 MB L2 beside the activation
+// panels in flight, so they get about 2.4 MB; every group re-reads the activations once, so
+// the groups are as few and as even as that allows.  Panels too long for two of them to fit
+// (large K) keep the plain column-fastest order.
+inline int column_group(int tiles_n, int bn, int Kp) {
+  const int64_t panel = (int64_t)bn * Kp * 2;
+  const int fit = (int)((2400 << 10) / panel);
+  if (fit < 2 || tiles_n <= fit) return tiles_n;
+  const int groups = (tiles_n + fit - 1) / fit;
+  return (tiles_n + groups - 1) / groups;
+}
+
 template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
 int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                hipStream_t st) {
@@ -474,21 +542,25 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
     attr_done = true;
   }
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (N + BN - 1) / BN;
+  int group_w = column_group(tiles_n, BN, Kp);
+#ifdef GPTMI_TUNING
+  if (g_group_w > 0) group_w = g_group_w < tiles_n ? g_group_w : tiles_n;
+#endif
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(WM * WN * 64), smem, st,
                      (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n,
-                     ep);
+                     group_w, ep);
   return 0;
 }
 
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
-  // Big problems: 256x256 tiles, 8 wavefronts (4x2, wave tile 64x128), K step 64 -- full
+  // Big problems: 256x256 tiles, 8 wavefronts (2x4, wave tile 128x64), K step 64 -- full
   // 128-byte rows per direct load move ~1.5x the bytes per clock of 64-byte rows -- double
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256)
-    return launch_cfg<256, 256, 4, 2, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+    return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 
