@@ -28,9 +28,10 @@ BATCH, SEQLEN = 512, 300
 ARCH = dict(vocab_size=50257, block_size=1024, n_layer=12, n_head=12, n_embd=768)
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 FFN1 = dict(M=BATCH * SEQLEN, N=3072, K=768)
-# HBM bytes of one ffn1 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/gemm_ffn1_pmc.md); None until measured for the shipped kernel
-FFN1_TRAFFIC_BYTES = None
+# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (890.7 MB after scaling by
+# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.7 MB); the counters cannot be read
+# from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
+FFN1_TRAFFIC_BYTES = 1.834e9
 
 
 def forward_flops(tokens, seqlen):
