@@ -168,7 +168,7 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
  *
  * Replaces flash_attention_v1(q, k, v, dropout_prob) -> kernels.py:477-525 and
  * flash_attention_v1_kernel -> kernels.py:375-474.
- *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64 or 128    Lq == Lk
+ *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64, 128 or 256    Lq == Lk
  *   out: [B][N][Lq][d] (GPTMI_O_BNLD) or [B][Lq][N][d] (GPTMI_O_BLND)
  * p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
  */
