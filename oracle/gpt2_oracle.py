@@ -16,6 +16,8 @@ operands in fp32 plus acc, casts = ndarray.astype, exp = np.exp):
   matmul_and_split_qkv  kernels.py:347-367
   flash_attention_v1    kernels.py:375-525
   softmax_rows          (dead sketch kernels.py:318-342; contract = softmax(x.float(), -1))
+  dropout / tl_rand     kernels.py:31-34 over Triton's tl.rand (triton/language/random.py:
+                        Philox-4x32-10, counter (offset,0,0,0), key = 64-bit seed, first word)
   gpt2_forward          gpt.py:38-60, 90-111, 163-180 (+ optional tied LM head,
                         the intent commented at gpt.py:159-161, 172-179)
 
@@ -33,6 +35,11 @@ What pins each function (tests/test_oracle.py):
                flash_attention_v1 under Triton's CPU interpreter (bit-identical on
                > 95 % of the elements, <= 2e-7 relative on the rest)
   softmax      torch.softmax in fp64
+  dropout      Philox-4x32-10 against the three known-answer vectors of the Random123
+               distribution (counter/key all zero, all ones, digits of pi), the uniform map
+               against its closed form on the int32 edge values, the keep rate against p, and
+               tests/golden/dropout.npz: outputs of the reference's fused_embeddings, fused_ffn
+               and flash_attention_v1 with dropout_prob > 0 under Triton's CPU interpreter
   model        an independently written fp64 torch GPT-2 (HF block order)
 No function of this file is left unpinned.
 """
@@ -54,13 +61,64 @@ def round_to_f16(a):
     return np.asarray(a).astype(F16).astype(F32)
 
 
-def fused_embeddings(ids, wte, wpe):
-    """kernels.py:58-70 with dropout_prob = 0: one add in the storage dtype."""
+U32 = np.uint32
+SEED = 1337  # the default of every kernel's `seed` argument (kernels.py:49,181,387)
+
+
+def philox4x32_10(c0, c1, c2, c3, k0, k1):
+    """Ten rounds of Philox-4x32 (triton/language/random.py:13-43); uint32 arrays in and out."""
+    c0, c1, c2, c3 = (np.asarray(c, dtype=U32).copy() for c in (c0, c1, c2, c3))
+    k0, k1 = int(k0) & 0xFFFFFFFF, int(k1) & 0xFFFFFFFF
+    A, B = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    for _ in range(10):
+        pa = A * c0.astype(np.uint64)  # 64-bit products: hi word = umulhi, lo word = mul
+        pb = B * c2.astype(np.uint64)
+        n0 = (pb >> np.uint64(32)).astype(U32) ^ c1 ^ U32(k0)
+        n2 = (pa >> np.uint64(32)).astype(U32) ^ c3 ^ U32(k1)
+        c1 = (pb & np.uint64(0xFFFFFFFF)).astype(U32)
+        c3 = (pa & np.uint64(0xFFFFFFFF)).astype(U32)
+        c0, c2 = n0, n2
+        k0 = (k0 + 0x9E3779B9) & 0xFFFFFFFF
+        k1 = (k1 + 0xBB67AE85) & 0xFFFFFFFF
+    return c0, c1, c2, c3
+
+
+def uint_to_uniform_float(x):
+    """triton/language/random.py:88-105: the word as int32, negatives folded by -x-1, times
+    4.6566127342e-10 in fp32 -> [0, 1)."""
+    xi = np.asarray(x, dtype=U32).view(np.int32)
+    xi = np.where(xi < 0, -xi - 1, xi)
+    return xi.astype(F32) * F32(4.6566127342e-10)
+
+
+def tl_rand(seed, offset):
+    """tl.rand(seed, offset) for 32-bit offsets (random.py:46-69,108-117)."""
+    off = np.asarray(offset).astype(np.int64).astype(U32)  # int32 offsets reinterpreted
+    zero = np.zeros_like(off)
+    c0, _, _, _ = philox4x32_10(off, zero, zero, zero, seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
+    return uint_to_uniform_float(c0)
+
+
+def dropout(x, p, seed, offset):
+    """kernels.py:31-34: keep where rand > p, scaled by a true division by (1 - p); the
+    arithmetic is fp32 (p is an fp32 scalar on the device)."""
+    keep = tl_rand(seed, offset) > F32(p)
+    return np.where(keep, _as_f32(x) / (F32(1.0) - F32(p)), F32(0.0)).astype(F32)
+
+
+def fused_embeddings(ids, wte, wpe, dropout_prob=0.0, seed=SEED):
+    """kernels.py:58-70: one add in the storage dtype, then dropout -- applied even at p = 0
+    (kernels.py:70), with the COLUMN index as the only offset (kernels.py:65), so the mask is
+    the same for every token.  At p = 0 a column would be zeroed only if its rand were exactly
+    0; the tests check that no column below 2^20 has that for the default seed."""
     ids = np.asarray(ids)
     B, L = ids.shape
     assert wte.shape[1] == wpe.shape[1] and wte.dtype == wpe.dtype
     pos = np.arange(B * L) % L  # kernels.py:61 -- position = pid % L
     rows = wte[ids.reshape(-1)] + wpe[pos]  # numpy adds fp16 + fp16 with one rounding
+    rows = rows.astype(wte.dtype, copy=False)
+    if dropout_prob != 0.0:
+        rows = dropout(rows, dropout_prob, seed, np.arange(wte.shape[1])[None, :])
     return rows.reshape(B, L, wte.shape[1]).astype(wte.dtype, copy=False)
 
 
@@ -90,8 +148,9 @@ def gelu_new(x):
     return F32(0.5) * x * (F32(1.0) + t)
 
 
-def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False):
-    """kernels.py:224-257: fp16 operands, fp32 accumulate, bias -> GELU -> residual -> cast."""
+def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False, dropout_prob=0.0, seed=SEED):
+    """kernels.py:224-257: fp16 operands, fp32 accumulate, bias -> GELU -> dropout (only if
+    p > 0, offset = flat index m*N + n in int32, kernels.py:245-251) -> residual -> cast."""
     out_dtype = x.dtype
     K = x.shape[-1]
     N = weight.shape[1]
@@ -103,6 +162,10 @@ def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False):
         z = z + _as_f32(bias)
     if add_gelu:
         z = gelu_new(z)
+    if dropout_prob > 0.0:
+        M = z.shape[0]
+        flat = (np.arange(M, dtype=np.int64)[:, None] * N + np.arange(N, dtype=np.int64)[None, :])
+        z = dropout(z, dropout_prob, seed, flat & 0xFFFFFFFF)
     if residual is not None:
         z = z + _as_f32(residual).reshape(z.shape)
     return z.astype(out_dtype).reshape(*x.shape[:-1], N)
@@ -123,8 +186,10 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
     return tuple(parts)
 
 
-def flash_attention_v1(q, k, v, block=BLOCK_L):
-    """kernels.py:408-474, dropout_prob = 0, Lq == Lk.
+def flash_attention_v1(q, k, v, block=BLOCK_L, dropout_prob=0.0, seed=SEED):
+    """kernels.py:408-474, Lq == Lk.  Dropout (p > 0 only) hits P after the denominator has
+    summed it and before the fp16 rounding, offset = lq * Lk + lk for every batch and head
+    (kernels.py:457-460).
 
     Per query row: key tiles of `block` in ascending order; S = (q16 . k16^T) * scale in
     fp32; causal mask; running max m; P = exp(S - m_new); den = den * exp(m - m_new) +
@@ -153,6 +218,8 @@ def flash_attention_v1(q, k, v, block=BLOCK_L):
             p = np.exp(s - mnew)
             mult = np.exp(mrun - mnew)
         den = den * mult + p.sum(axis=2, dtype=F32, keepdims=True)
+        if dropout_prob > 0.0:
+            p = dropout(p, dropout_prob, seed, (rows * L + cols)[None])
         acc = acc * mult + np.matmul(round_to_f16(p), v16[:, k0:k1], dtype=F32)
         mrun = mnew
     out = acc / den

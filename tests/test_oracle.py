@@ -2,6 +2,7 @@
 routines, fp64 closed forms, invariants and special cases chosen so that a dropped term, a
 wrong sign/index or a transposed operand fails.  No GPU involved."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -343,3 +344,100 @@ def test_model_composition_vs_independent_fp64_gpt2():
     bad["blocks.1.1.ffn2_bias"] = -params["blocks.1.1.ffn2_bias"]
     bad_h = O.gpt2_forward(bad, ids, cfg["n_head"])
     assert np.abs(bad_h - want_h).max() > 2e-2 * np.abs(want_h).max()
+
+
+# ---------------------------------------------------------------------------
+# dropout: Philox-4x32-10 -> tl.rand -> keep mask (kernels.py:31-34)
+# ---------------------------------------------------------------------------
+PHILOX_KAT = [  # counter, key, output: the philox4x32 10-round vectors of the Random123 distribution
+    ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+    ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+    ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+     (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+]
+
+
+@pytest.mark.parametrize("ctr,key,want", PHILOX_KAT)
+def test_philox_known_answers(ctr, key, want):
+    got = O.philox4x32_10(*[np.array([c], dtype=np.uint32) for c in ctr], *key)
+    assert tuple(int(g[0]) for g in got) == want
+
+
+def test_philox_is_elementwise():
+    offs = np.array([0, 1, 2, 0xFFFFFFFF, 12345], dtype=np.uint32)
+    z = np.zeros_like(offs)
+    whole = O.philox4x32_10(offs, z, z, z, 1337, 0)[0]
+    single = [O.philox4x32_10(offs[i:i + 1], z[:1], z[:1], z[:1], 1337, 0)[0][0] for i in range(5)]
+    assert whole.tolist() == single
+    assert len(set(whole.tolist())) == 5
+
+
+def test_uniform_map_closed_form():
+    # int32 view, negatives folded by -x-1, times 4.6566127342e-10 in fp32
+    words = np.array([0, 1, 0x7FFFFFFF, 0x80000000, 0xFFFFFFFF, 0x40000000], dtype=np.uint32)
+    want = np.array([0, 1, 2**31 - 1, 2**31 - 1, 0, 2**30], dtype=np.float64)
+    got = O.uint_to_uniform_float(words)
+    assert got.dtype == np.float32
+    assert np.array_equal(got, (want.astype(np.float32) * np.float32(4.6566127342e-10)))
+    assert got.max() < 1.0 and got.min() == 0.0
+
+
+def test_rand_default_seed_statistics_and_no_exact_zero():
+    r = O.tl_rand(1337, np.arange(1 << 20))
+    # the embedding applies dropout even at p = 0 (kernels.py:70): identity iff rand > 0
+    assert (r > 0).all() and (r < 1).all()
+    assert abs(r.mean() - 0.5) < 2e-3
+    for p in (0.1, 0.25, 0.5):
+        assert abs((r > np.float32(p)).mean() - (1 - p)) < 2e-3
+    # seeds and offsets are distinct streams
+    assert not np.array_equal(r[:64], O.tl_rand(1338, np.arange(64)))
+    # int32 offsets wrap like the device's: -1 is counter 0xFFFFFFFF
+    assert O.tl_rand(1337, np.array([-1]))[0] == O.tl_rand(1337, np.array([0xFFFFFFFF]))[0]
+
+
+def test_dropout_scales_by_true_division():
+    x = rng(5).standard_normal((4, 50)).astype(np.float32)
+    off = np.arange(200).reshape(4, 50)
+    y = O.dropout(x, 0.3, 1337, off)
+    keep = O.tl_rand(1337, off) > np.float32(0.3)
+    assert np.array_equal(y[keep], x[keep] / (np.float32(1) - np.float32(0.3)))
+    assert (y[~keep] == 0).all() and 0.55 < keep.mean() < 0.85
+
+
+def _golden_dropout():
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "dropout.npz"))
+    return g, (lambda k: g[k].astype(np.float32))
+
+
+def test_dropout_embeddings_vs_reference_golden_vectors():
+    """tests/golden/dropout.npz: outputs of the reference's own operators with dropout under
+    Triton's CPU interpreter (tests/golden/make_dropout_vectors.py)."""
+    g, f = _golden_dropout()
+    got = O.fused_embeddings(g["emb_ids"], f("emb_wte"), f("emb_wpe"), dropout_prob=float(g["emb_p"]))
+    assert np.array_equal(got, g["emb_out"])
+    # one mask for all tokens: the zero pattern is a function of the column alone
+    zero = g["emb_out"] == 0
+    assert (zero == zero[0, 0]).all() and 0 < zero[0, 0].mean() < 0.5
+    assert np.array_equal(O.fused_embeddings(g["emb_ids"], f("emb_wte"), f("emb_wpe")), g["emb_out_p0"])
+
+
+def test_dropout_ffn_vs_reference_golden_vectors():
+    g, f = _golden_dropout()
+    got = O.fused_ffn(f("ffn_x"), f("ffn_w"), bias=f("ffn_b"), residual=f("ffn_r"), add_gelu=True,
+                      dropout_prob=float(g["ffn_p"]))
+    assert np.abs(got - g["ffn_out"]).max() <= 4e-6  # summation order of the fp32 products
+    # where the value was dropped the output is the residual itself: pins dropout-before-residual
+    dropped = g["ffn_out"] == f("ffn_r")
+    assert 0.05 < dropped.mean() < 0.16 and np.array_equal(dropped, got == f("ffn_r"))
+    plain = O.fused_ffn(f("ffn_x"), f("ffn_w"), dropout_prob=0.5)
+    assert np.array_equal(plain == 0, g["ffn_out_plain"] == 0)
+    assert np.abs(plain - g["ffn_out_plain"]).max() <= 4e-6
+
+
+def test_dropout_attention_vs_reference_golden_vectors():
+    g, f = _golden_dropout()
+    got = O.flash_attention_v1(f("att_q"), f("att_k"), f("att_v"), dropout_prob=float(g["att_p"]))
+    d = np.abs(got - g["att_out"])
+    assert d.max() <= 2e-6 * np.abs(g["att_out"]).max() and (d == 0).mean() > 0.95
+    # and it is not the p = 0 result
+    assert np.abs(O.flash_attention_v1(f("att_q"), f("att_k"), f("att_v")) - g["att_out"]).max() > 0.05
