@@ -29,6 +29,7 @@ static int check_launch(const char* what) {
 }
 
 static bool dtype_ok(int dtype) { return dtype == GPTMI_F32 || dtype == GPTMI_F16; }
+static bool dropout_ok(float p) { return p >= 0.0f && p < 1.0f; }  // false for NaN too
 
 static inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
@@ -104,7 +105,6 @@ const char* gptmi_last_error(void) { return g_err; }
 int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out, int64_t B,
                 int64_t L, int64_t V, int64_t P, int64_t H, float p, uint64_t seed,
                 int dtype, void* stream) {
-  (void)seed;
   if (!ids || !wte || !wpe || !out || B <= 0 || L <= 0 || V <= 0 || P <= 0 || H <= 0 ||
       !dtype_ok(dtype)) {
     set_error("embed: invalid argument");
@@ -119,11 +119,12 @@ int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
     set_error("embed: H=%lld too large", (long long)H);
     return GPTMI_ERR_UNSUPPORTED;
   }
-  if (p != 0.0f) {
-    set_error("embed: dropout (p=%g) is not implemented", (double)p);
-    return GPTMI_ERR_UNSUPPORTED;
+  if (!dropout_ok(p)) {
+    set_error("embed: dropout probability %g outside [0, 1)", (double)p);
+    return GPTMI_ERR_INVALID;
   }
-  launch_embed(ids, wte, wpe, out, B * L, L, (int)H, dtype == GPTMI_F16, (hipStream_t)stream);
+  launch_embed(ids, wte, wpe, out, B * L, L, (int)H, Dropout{p, seed}, dtype == GPTMI_F16,
+               (hipStream_t)stream);
   return check_launch("embed");
 }
 
@@ -187,7 +188,6 @@ int gptmi_linear(const void* x, const void* W, const void* bias, const void* res
                  void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
                  uint64_t seed, int wlayout, void* workspace, size_t workspace_bytes,
                  int dtype, void* stream) {
-  (void)seed;
   if (!x || !W || !out || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
       (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK && wlayout != GPTMI_W_PACKED)) {
     set_error("linear: invalid argument");
@@ -197,9 +197,9 @@ int gptmi_linear(const void* x, const void* W, const void* bias, const void* res
     set_error("linear: N or K too large");
     return GPTMI_ERR_UNSUPPORTED;
   }
-  if (p != 0.0f) {
-    set_error("linear: dropout (p=%g) is not implemented", (double)p);
-    return GPTMI_ERR_UNSUPPORTED;
+  if (!dropout_ok(p)) {
+    set_error("linear: dropout probability %g outside [0, 1)", (double)p);
+    return GPTMI_ERR_INVALID;
   }
   hipStream_t st = (hipStream_t)stream;
   const void *A, *Bt;
@@ -216,6 +216,7 @@ int gptmi_linear(const void* x, const void* W, const void* bias, const void* res
   ep.residual = residual;
   ep.out = out;
   ep.gelu = gelu ? 1 : 0;
+  ep.drop = Dropout{p, seed};
   ep.qkv = false;
   ep.f16 = dtype == GPTMI_F16;
   rc = launch_gemm(A, Bt, M, (int)N, Kp, ep, st);
@@ -269,7 +270,6 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, vo
 int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int64_t B,
                      int64_t N, int64_t Lq, int64_t Lk, int64_t d, float scale, float p,
                      uint64_t seed, int olayout, int dtype, void* stream) {
-  (void)seed;
   if (!q || !k || !v || !out || B <= 0 || N <= 0 || Lq <= 0 || Lk <= 0 || d <= 0 ||
       !dtype_ok(dtype) || (olayout != GPTMI_O_BNLD && olayout != GPTMI_O_BLND)) {
     set_error("flash_attn: invalid argument");
@@ -281,16 +281,17 @@ int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int
               (long long)Lq, (long long)Lk);
     return GPTMI_ERR_UNSUPPORTED;
   }
-  if (p != 0.0f) {
-    set_error("flash_attn: dropout (p=%g) is not implemented", (double)p);
-    return GPTMI_ERR_UNSUPPORTED;
+  if (!dropout_ok(p)) {
+    set_error("flash_attn: dropout probability %g outside [0, 1)", (double)p);
+    return GPTMI_ERR_INVALID;
   }
   if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) ||
       ((uintptr_t)out & 15)) {
     set_error("flash_attn: q, k, v and out must be 16-byte aligned");
     return GPTMI_ERR_INVALID;
   }
-  int rc = launch_flash_attn(q, k, v, out, B, N, Lq, (int)d, scale, olayout == GPTMI_O_BLND,
+  int rc = launch_flash_attn(q, k, v, out, B, N, Lq, (int)d, scale, Dropout{p, seed},
+                             olayout == GPTMI_O_BLND,
                              dtype == GPTMI_F16, (hipStream_t)stream);
   if (rc) return rc;
   return check_launch("flash_attn");

@@ -68,10 +68,10 @@ __device__ __forceinline__ h8 zero_h8() {
 // D = head size.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
 // position c ^ (r&7)) and V^T tile [D][64] (8-byte unit u of row d at position
 // u ^ ((d>>1)&15)).
-template <int D, typename T, bool BLND>
+template <int D, typename T, bool BLND, bool DROP>
 __global__ __launch_bounds__(256) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-    T* __restrict__ O, int heads, int L, float scale) {
+    T* __restrict__ O, int heads, int L, float scale, DropoutArgs drop) {
   constexpr int CH = D / 8;             // 16-byte chunks per row
   constexpr int KS = D / 16;            // MFMA k-steps over the head dim
   constexpr int DB = D / 32;            // 32-row blocks of O^T
@@ -227,6 +227,22 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
       psum += __shfl_xor(psum, 32, kWave);
       den = den * mult + psum;
       mrun = mnew;
+      if constexpr (DROP) {
+        // dropout of P after the denominator has summed it, before the fp16 rounding;
+        // offset = query * L + key, the same for every batch and head (kernels.py:457-460)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const unsigned key0 = (unsigned)(k0 + kb * 32 + 8 * rg + 4 * g);
+            const unsigned base_off = (unsigned)q * (unsigned)L + key0;
+            unsigned off[4] = {base_off, base_off + 1u, base_off + 2u, base_off + 3u};
+            float pv[4] = {s[kb][4 * rg], s[kb][4 * rg + 1], s[kb][4 * rg + 2], s[kb][4 * rg + 3]};
+            dropout_apply<4>(drop, off, pv);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[kb][4 * rg + e] = pv[e];
+          }
+      }
 #pragma unroll
       for (int i = 0; i < DB; ++i)
 #pragma unroll
@@ -538,46 +554,50 @@ int launch_resident(const void* q, const void* k, const void* v, void* out, int6
   return 0;
 }
 
-template <int D, typename T>
-int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
-             int heads, int L, float scale, bool blnd, hipStream_t st) {
-  if (const size_t lds = resident_lds_bytes(L, D)) {
-    return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
-                : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
-  }
+template <int D, typename T, bool BLND, bool DROP>
+int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                 int L, float scale, DropoutArgs drop, hipStream_t st) {
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
   constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V^T tile
-  auto k_blnd = flash_attn_kernel<D, T, true>;
-  auto k_bnld = flash_attn_kernel<D, T, false>;
-  static bool attr_done = false;  // idempotent; a race only repeats the calls
+  auto kern = flash_attn_kernel<D, T, BLND, DROP>;
+  static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_blnd),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_bnld),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) {
       set_error("hipFuncSetAttribute(%d bytes LDS): %s", lds, hipGetErrorString(e));
       return -4;
     }
   }
   attr_done = true;
-  if (blnd)
-    hipLaunchKernelGGL(k_blnd, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
-                       (T*)out, heads, L, scale);
-  else
-    hipLaunchKernelGGL(k_bnld, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
-                       (T*)out, heads, L, scale);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
+                     (T*)out, heads, L, scale, drop);
   return 0;
+}
+
+template <int D, typename T>
+int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
+             int heads, int L, float scale, Dropout drop, bool blnd, hipStream_t st) {
+  const DropoutArgs da = {drop.p, (unsigned)drop.seed, (unsigned)(drop.seed >> 32)};
+  if (drop.p > 0.f) {  // training-mode path: the tiled kernel carries the generator
+    return blnd ? launch_tiled<D, T, true, true>(q, k, v, out, BN, heads, L, scale, da, st)
+                : launch_tiled<D, T, false, true>(q, k, v, out, BN, heads, L, scale, da, st);
+  }
+  if (const size_t lds = resident_lds_bytes(L, D)) {
+    return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
+                : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
+  }
+  return blnd ? launch_tiled<D, T, true, false>(q, k, v, out, BN, heads, L, scale, da, st)
+              : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, scale, da, st);
 }
 
 template <typename T>
 int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
-             int heads, int L, int d, float scale, bool blnd, hipStream_t st) {
+             int heads, int L, int d, float scale, Dropout drop, bool blnd, hipStream_t st) {
   switch (d) {
-    case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
-    case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
-    case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, scale, blnd, st);
+    case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
+    case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
+    case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
     default:
       set_error("flash_attn: head size %d not built (64, 128 and 256 are)", d);
       return -2;
@@ -587,16 +607,16 @@ int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
 }  // namespace
 
 int launch_flash_attn(const void* q, const void* k, const void* v, void* out, int64_t B,
-                      int64_t N, int64_t L, int d, float scale, bool out_blnd, bool f16,
-                      hipStream_t st) {
+                      int64_t N, int64_t L, int d, float scale, Dropout drop, bool out_blnd,
+                      bool f16, hipStream_t st) {
   const int64_t BN = B * N;
   if (BN > 0x7fffffffll || L > (1 << 24)) {
     set_error("flash_attn: B*N=%lld or L=%lld beyond the grid limits", (long long)BN,
               (long long)L);
     return -2;
   }
-  return f16 ? launch_t<_Float16>(q, k, v, out, BN, (int)N, (int)L, d, scale, out_blnd, st)
-             : launch_t<float>(q, k, v, out, BN, (int)N, (int)L, d, scale, out_blnd, st);
+  return f16 ? launch_t<_Float16>(q, k, v, out, BN, (int)N, (int)L, d, scale, drop, out_blnd, st)
+             : launch_t<float>(q, k, v, out, BN, (int)N, (int)L, d, scale, drop, out_blnd, st);
 }
 
 }  // namespace gptmi

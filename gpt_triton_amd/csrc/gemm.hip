@@ -50,6 +50,7 @@ struct EpiDev {
   int d;
   int gelu;
   int vec_ok;  // pointers and N allow 4-element vector accesses
+  DropoutArgs drop;  // p > 0: dropout between GELU and residual (predicated epilogue only)
 #ifdef GPTMI_TUNING
   unsigned long long* trace;  // tuning builds only: per-workgroup phase time stamps
 #endif
@@ -131,7 +132,7 @@ constexpr int EP_SLAB = 32 * EP_STRIDE; // one wavefront's staging slab
 // (fp16) or 256-byte (fp32) runs per row.
 //   FAST: the workgroup tile lies entirely inside M x N and every pointer
 //   allows 4-element vector accesses -- straight-line code, no predicates.
-template <int MB, int NB, typename T, bool QKV, bool FAST, bool GELU, bool RES>
+template <int MB, int NB, typename T, bool QKV, bool FAST, bool GELU, bool RES, bool DROP = false>
 __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const EpiDev& ep,
                                                   int64_t mw0, int nw0, int M, int N, char* slab,
                                                   int lane) {
@@ -207,7 +208,7 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
           *reinterpret_cast<f4*>(slab + frow * EP_STRIDE + (ii * 32 + g * 8 + fhalf * 4) * 4) = z;
         }
       }
-#pragma unroll
+#pragma unroll(DROP ? 1 : 8)
       for (int rr = 0; rr < 8; ++rr) {
         const int row = rr * 4 + rrow;
         const int64_t m = mbase + row;
@@ -248,6 +249,15 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
           if (m >= M || n >= N) continue;
           T* op = out_ptr<T, QKV>(ep, m, n, N);
           const T* rp = RES ? (const T*)ep.residual + (m * (int64_t)N + n) : nullptr;
+          if constexpr (DROP) {
+            // the generator's offset is the flat index m*N + n in 32 bits (kernels.py:245)
+            const unsigned flat = (unsigned)((uint64_t)m * (uint64_t)N + (uint64_t)n);
+            unsigned off[4] = {flat, flat + 1u, flat + 2u, flat + 3u};
+            float zz[4] = {z[0], z[1], z[2], z[3]};
+            dropout_apply<4>(ep.drop, off, zz);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) z[e] = zz[e];
+          }
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (n + e < N) op[e] = (T)(z[e] + (RES ? (float)rp[e] : 0.f));
@@ -262,6 +272,16 @@ __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDe
                                                 int64_t mw0, int nw0, int M, int N, bool fast,
                                                 char* slab, int lane) {
   const bool res = !QKV && ep.residual != nullptr;
+  if constexpr (!QKV) {
+    if (ep.drop.p > 0.f) {  // training-mode path: always the predicated variant
+#define GPTMI_EPI_DROP(G, R) \
+  store_wave_tile_v<MB, NB, T, QKV, false, G, R, true>(acc, ep, mw0, nw0, M, N, slab, lane)
+      if (ep.gelu) { if (res) GPTMI_EPI_DROP(true, true); else GPTMI_EPI_DROP(true, false); }
+      else { if (res) GPTMI_EPI_DROP(false, true); else GPTMI_EPI_DROP(false, false); }
+#undef GPTMI_EPI_DROP
+      return;
+    }
+  }
 #define GPTMI_EPI(F, G, R) \
   store_wave_tile_v<MB, NB, T, QKV, F, G, R>(acc, ep, mw0, nw0, M, N, slab, lane)
   if (fast) {
@@ -588,6 +608,8 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const G
   ep.heads = e.heads;
   ep.d = e.d;
   ep.gelu = e.gelu;
+  ep.drop = DropoutArgs{e.qkv ? 0.f : e.drop.p, (unsigned)e.drop.seed,
+                        (unsigned)(e.drop.seed >> 32)};
   const uintptr_t amask = e.f16 ? 7 : 15;
   auto aligned = [&](const void* p) { return p == nullptr || ((uintptr_t)p & amask) == 0; };
   const bool vec = (N % 4) == 0 && aligned(e.bias) && aligned(e.residual) && aligned(e.out) &&

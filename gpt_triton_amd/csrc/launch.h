@@ -6,8 +6,14 @@
 
 namespace gptmi {
 
+// Dropout of one launch: probability p (0 = none) and the 64-bit seed of the generator.
+struct Dropout {
+  float p;
+  uint64_t seed;
+};
+
 int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
-                 int64_t rows, int64_t L, int H, bool f16, hipStream_t st);
+                 int64_t rows, int64_t L, int H, Dropout drop, bool f16, hipStream_t st);
 int launch_layernorm(const void* x, const void* w, const void* b, void* out,
                      int64_t M, int H, float eps, bool f16, hipStream_t st);
 int launch_softmax(const void* x, void* out, int64_t M, int H, bool f16,
@@ -30,6 +36,7 @@ struct GemmEpilogue {
   int heads;      // qkv mode
   int d;          // qkv mode: head size
   int gelu;       // apply tanh-GELU after the bias
+  Dropout drop;   // after the GELU, before the residual (plain mode only)
   bool qkv;       // scatter mode
   bool f16;       // storage dtype of bias / residual / outputs
 };
@@ -40,7 +47,7 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
                 const GemmEpilogue& ep, hipStream_t st);
 
 int launch_flash_attn(const void* q, const void* k, const void* v, void* out,
-                      int64_t B, int64_t N, int64_t L, int d, float scale,
+                      int64_t B, int64_t N, int64_t L, int d, float scale, Dropout drop,
                       bool out_blnd, bool f16, hipStream_t st);
 
 }  // namespace gptmi

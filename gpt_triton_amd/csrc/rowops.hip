@@ -57,6 +57,28 @@ __global__ __launch_bounds__(256) void embed_scalar_kernel(
     out[row * H + c] = (T)((float)wte[tok * H + c] + (float)wpe[pos * H + c]);
 }
 
+// Embedding with dropout (kernels.py:65-70): the sum is rounded to the storage dtype first,
+// the dropout works on that value in fp32 with the COLUMN as the generator's offset, so every
+// token sees the same mask.  Training-mode path: one Philox evaluation per element.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_dropout_kernel(
+    const int64_t* __restrict__ ids, const T* __restrict__ wte,
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H,
+    DropoutArgs drop) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t tok = ids[row];
+  const int64_t pos = row % L;
+  for (int c = lane; c < H; c += 64) {
+    const T sum = (T)((float)wte[tok * H + c] + (float)wpe[pos * H + c]);
+    unsigned off[1] = {(unsigned)c};
+    float z[1] = {(float)sum};
+    dropout_apply<1>(drop, off, z);
+    out[row * H + c] = (T)z[0];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // LayerNorm (reference: fused_layer_norm_kernel, kernels.py:104-145): fp32
 // mean, then fp32 centred biased variance, rstd = 1/sqrt(var + eps),
@@ -264,9 +286,18 @@ __global__ __launch_bounds__(256) void pack_transpose_kernel(const T* __restrict
 // ---------------------------------------------------------------------------
 template <typename T>
 static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
-                          void* out, int64_t rows, int64_t L, int H,
+                          void* out, int64_t rows, int64_t L, int H, Dropout drop,
                           hipStream_t st) {
   const unsigned grid = (unsigned)((rows + 3) / 4);
+  // The reference runs the dropout even at p = 0 (kernels.py:70), where it is the identity
+  // unless a column's uniform is exactly 0; for the default seed no column below 2^20 has
+  // that, so only other seeds or wider rows need the generator at p = 0.
+  if (drop.p != 0.0f || drop.seed != 1337 || H > (1 << 20)) {
+    const DropoutArgs d = {drop.p, (unsigned)drop.seed, (unsigned)(drop.seed >> 32)};
+    hipLaunchKernelGGL(embed_dropout_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
+                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H, d);
+    return 0;
+  }
   const bool aligned = (H % Vec<T>::N) == 0 && ((uintptr_t)wte % 16) == 0 &&
                        ((uintptr_t)wpe % 16) == 0 && ((uintptr_t)out % 16) == 0;
   if (aligned)
@@ -279,9 +310,9 @@ static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
 }
 
 int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
-                 int64_t rows, int64_t L, int H, bool f16, hipStream_t st) {
-  return f16 ? launch_embed_t<_Float16>(ids, wte, wpe, out, rows, L, H, st)
-             : launch_embed_t<float>(ids, wte, wpe, out, rows, L, H, st);
+                 int64_t rows, int64_t L, int H, Dropout drop, bool f16, hipStream_t st) {
+  return f16 ? launch_embed_t<_Float16>(ids, wte, wpe, out, rows, L, H, drop, st)
+             : launch_embed_t<float>(ids, wte, wpe, out, rows, L, H, drop, st);
 }
 
 template <typename T, int CH>

@@ -13,8 +13,11 @@ plus `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:3
 `lm_head(x, wte)` (the transposed-weight product the reference leaves as a TODO,
 gpt.py:159-161) and `pack_weight(weight)`: the GEMM reads its weight as an fp16,
 K-contiguous image which `fused_ffn` / `matmul_and_split_qkv` otherwise rebuild on every
-call; a `PackedWeight` may be passed wherever they take `weight`.  Tensors must live on the GPU: there is no CPU path.  dropout_prob > 0
-raises NotImplementedError.
+call; a `PackedWeight` may be passed wherever they take `weight`.  Tensors must live on the
+GPU: there is no CPU path.  dropout_prob > 0 reproduces the reference's masks: Philox-4x32-10
+(Triton's tl.rand) with the kernels' default seed 1337 and the reference's offsets -- the column
+for the embedding, the flat index m*N + n for fused_ffn, query*Lk + key for the attention
+weights (kernels.py:31-34, 65-70, 245-251, 457-460).
 """
 import math
 

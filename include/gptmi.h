@@ -38,7 +38,7 @@ typedef enum gptmi_dtype {
 
 typedef enum gptmi_status {
   GPTMI_OK = 0,
-  GPTMI_ERR_INVALID = -1,     /* NULL pointer, non-positive size, bad enum */
+  GPTMI_ERR_INVALID = -1,     /* NULL pointer, non-positive size, bad enum, p outside [0,1) */
   GPTMI_ERR_UNSUPPORTED = -2, /* valid request the kernels do not implement */
   GPTMI_ERR_WORKSPACE = -3,   /* workspace missing or too small */
   GPTMI_ERR_LAUNCH = -4       /* hipGetLastError() after the launch != success */
@@ -71,8 +71,13 @@ const char* gptmi_last_error(void);
  * fused_embeddings_kernel -> kernels.py:37-72.
  *   ids  int64 [B*L]          wte [V][H]     wpe [P][H]     out [B*L][H]
  * Requires L <= P.  Token ids are NOT range checked on the device (neither does
- * the reference); the host wrapper may check them.  p must be 0 (dropout is not
- * implemented: GPTMI_ERR_UNSUPPORTED); seed is accepted for signature stability.
+ * the reference); the host wrapper may check them.
+ * Dropout (0 <= p < 1, dropout() -> kernels.py:31-34): the sum, rounded to the storage
+ * dtype, is kept where rand(seed, column) > p and divided by (1 - p), else zeroed; rand is
+ * Triton's tl.rand, i.e. Philox-4x32-10 with counter (column, 0, 0, 0), the 64-bit seed as
+ * key and the first output word mapped to [0, 1).  The column is the only offset
+ * (kernels.py:65-70), so every token gets the same mask; the reference's seed is 1337
+ * (kernels.py:49).
  */
 int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
                 int64_t B, int64_t L, int64_t V, int64_t P, int64_t H,
@@ -136,7 +141,10 @@ int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wla
  *   bias [N] or NULL
  *   residual [M][N] or NULL     out [M][N]
  * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
- * (may be NULL when that is 0).  p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
+ * (may be NULL when that is 0).
+ * Dropout (0 < p < 1; 0 = none) sits between the GELU and the residual
+ * (kernels.py:245-255): keep where rand(seed, (uint32)(m*N + n)) > p, divide by (1 - p);
+ * same generator as gptmi_embed, reference seed 1337 (kernels.py:181).
  */
 int gptmi_linear(const void* x, const void* W, const void* bias,
                  const void* residual, void* out, int64_t M, int64_t N, int64_t K,
@@ -170,7 +178,9 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
  * flash_attention_v1_kernel -> kernels.py:375-474.
  *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64, 128 or 256    Lq == Lk
  *   out: [B][N][Lq][d] (GPTMI_O_BNLD) or [B][Lq][N][d] (GPTMI_O_BLND)
- * p must be 0 (GPTMI_ERR_UNSUPPORTED otherwise).
+ * Dropout (0 < p < 1; 0 = none) hits P after the denominator has summed it and before its
+ * fp16 rounding (kernels.py:457-466): keep where rand(seed, (uint32)(lq*Lk + lk)) > p,
+ * divide by (1 - p); the offset ignores batch and head, reference seed 1337 (kernels.py:387).
  */
 int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out,
                      int64_t B, int64_t N, int64_t Lq, int64_t Lk, int64_t d,

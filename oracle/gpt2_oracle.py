@@ -277,23 +277,29 @@ def n_layers_of(params):
     return 1 + max(int(k.split(".")[1]) for k in params if k.startswith("blocks."))
 
 
-def gpt2_forward(params, ids, n_head, lm_head=False):
-    """FusedGPT.forward in eval mode (gpt.py:163-180); every operator output is stored in
-    the parameter dtype, as it is between the reference's kernels."""
-    x = fused_embeddings(ids, params["wte_weight"], params["wpe_weight"])
+def gpt2_forward(params, ids, n_head, lm_head=False, dropout_prob=0.0):
+    """FusedGPT.forward (gpt.py:163-180); every operator output is stored in the parameter
+    dtype, as it is between the reference's kernels.  dropout_prob = 0 is eval mode; in
+    training mode the reference hands its dropout to the embedding, the attention weights,
+    the attention projection and BOTH ffn products (gpt.py:44-58, 92-109, 165-167)."""
+    p = dropout_prob
+    x = fused_embeddings(ids, params["wte_weight"], params["wpe_weight"], dropout_prob=p)
     for i in range(n_layers_of(params)):
         a, m = f"blocks.{i}.0.", f"blocks.{i}.1."
         res = x
         y = fused_layer_norm(x, params[a + "layer_norm_weight"], params[a + "layer_norm_bias"])
         q, k, v = matmul_and_split_qkv(y, params[a + "c_attn_weight"], params[a + "c_attn_bias"],
                                        n_head)
-        o = flash_attention_v1(q, k, v)
+        o = flash_attention_v1(q, k, v, dropout_prob=p)
         o = np.ascontiguousarray(o.transpose(0, 2, 1, 3)).reshape(res.shape)  # gpt.py:51
-        x = fused_ffn(o, params[a + "c_proj_weight"], bias=params[a + "c_proj_bias"], residual=res)
+        x = fused_ffn(o, params[a + "c_proj_weight"], bias=params[a + "c_proj_bias"], residual=res,
+                      dropout_prob=p)
         res = x
         y = fused_layer_norm(x, params[m + "layer_norm_weight"], params[m + "layer_norm_bias"])
-        y = fused_ffn(y, params[m + "ffn1_weight"], bias=params[m + "ffn1_bias"], add_gelu=True)
-        x = fused_ffn(y, params[m + "ffn2_weight"], bias=params[m + "ffn2_bias"], residual=res)
+        y = fused_ffn(y, params[m + "ffn1_weight"], bias=params[m + "ffn1_bias"], add_gelu=True,
+                      dropout_prob=p)
+        x = fused_ffn(y, params[m + "ffn2_weight"], bias=params[m + "ffn2_bias"], residual=res,
+                      dropout_prob=p)
     x = fused_layer_norm(x, params["layer_norm_weight"], params["layer_norm_bias"])
     if not lm_head:
         return x

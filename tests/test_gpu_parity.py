@@ -336,8 +336,8 @@ def test_operator_errors(K, gpu_device):
     with pytest.raises(AssertionError):
         q = torch.zeros((1, 1, 8, 48), device=gpu_device)  # head size not in the allowed set
         K.flash_attention_v1(q, q, q)
-    with pytest.raises(NotImplementedError):
-        K.fused_ffn(x, w, dropout_prob=0.1)
+    with pytest.raises(RuntimeError):
+        K.fused_ffn(x, w, dropout_prob=1.0)  # the keep scale 1 / (1 - p) does not exist
     with pytest.raises(TypeError):
         K.fused_ffn(x.double(), w.double())
 
@@ -492,3 +492,108 @@ def test_full_size_rowops(K, gpu_device):
           "softmax full size")
     # every softmax row sums to one (fp16 rounding of 768 terms)
     assert (sm.float().sum(dim=1) - 1).abs().max() < 2e-3
+
+
+# ----------------------------------------------------------------------------- dropout (p > 0)
+def _golden_dropout():
+    import os
+
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "dropout.npz"))
+    return g, (lambda k: g[k].astype(np.float32))
+
+
+def test_dropout_reference_golden_vectors(K, gpu_device):
+    """Outputs of the reference's own operators with dropout_prob > 0 (Triton CPU interpreter,
+    tests/golden/make_dropout_vectors.py): same masks, same place in each epilogue."""
+    g, f = _golden_dropout()
+    D = lambda a: dev(a, gpu_device)
+    z = K.fused_embeddings(D(g["emb_ids"]), D(f("emb_wte")), D(f("emb_wpe")),
+                           dropout_prob=float(g["emb_p"]))
+    assert np.array_equal(host(z), g["emb_out"])
+    z = K.fused_ffn(D(f("ffn_x")), D(f("ffn_w")), bias=D(f("ffn_b")), residual=D(f("ffn_r")),
+                    add_gelu=True, dropout_prob=float(g["ffn_p"]))
+    check(host(z), g["ffn_out"], torch.float32, "ffn")
+    assert np.array_equal(host(z) == f("ffn_r"), g["ffn_out"] == f("ffn_r"))  # the same mask
+    z = K.fused_ffn(D(f("ffn_x")), D(f("ffn_w")), dropout_prob=0.5)
+    assert np.array_equal(host(z) == 0, g["ffn_out_plain"] == 0)
+    check(host(z), g["ffn_out_plain"], torch.float32, "ffn plain")
+    z = K.flash_attention_v1(D(f("att_q")), D(f("att_k")), D(f("att_v")),
+                             dropout_prob=float(g["att_p"]))
+    check_attention(host(z), g["att_out"], f("att_v") / (1 - float(g["att_p"])), torch.float32,
+                    "attention")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("H", [96, 768, 1000])
+def test_dropout_embeddings(K, gpu_device, dtype, H):
+    r = np.random.default_rng(11)
+    ids = r.integers(0, 37, size=(5, 19))
+    wte = r.standard_normal((37, H)).astype(NP[dtype])
+    wpe = r.standard_normal((24, H)).astype(NP[dtype])
+    z = host(K.fused_embeddings(dev(ids, gpu_device), dev(wte, gpu_device), dev(wpe, gpu_device),
+                                dropout_prob=0.3))
+    want = O.fused_embeddings(ids, wte, wpe, dropout_prob=0.3)
+    if dtype == torch.float32:
+        assert np.array_equal(z, want)
+    else:  # one division in fp32 and one rounding on both sides
+        assert np.array_equal(z, want)
+    dropped = ~(O.tl_rand(1337, np.arange(H)) > np.float32(0.3))
+    assert (z[..., dropped] == 0).all() and 0.1 < dropped.mean() < 0.5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,K_,gelu,res", [(300, 520, 192, True, True), (2500, 300, 64, False, False),
+                                             (64, 1000, 100, True, False)])
+def test_dropout_ffn(K, gpu_device, dtype, M, N, K_, gelu, res):
+    """Both tile configurations (M >= 2048 takes the 256 x 256 one), ragged edges, p = 0.15."""
+    r = np.random.default_rng(12)
+    x = r.standard_normal((M, K_)).astype(NP[dtype])
+    w = (0.1 * r.standard_normal((K_, N))).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(N)).astype(NP[dtype])
+    rs = r.standard_normal((M, N)).astype(NP[dtype]) if res else None
+    z = host(K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device),
+                         residual=None if rs is None else dev(rs, gpu_device), add_gelu=gelu,
+                         dropout_prob=0.15))
+    want = O.fused_ffn(x, w, bias=b, residual=rs, add_gelu=gelu, dropout_prob=0.15)
+    check(z, want, dtype, "ffn dropout")
+    flat = np.arange(M, dtype=np.int64)[:, None] * N + np.arange(N)[None, :]
+    dropped = ~(O.tl_rand(1337, flat) > np.float32(0.15))
+    base = np.zeros((M, N), NP[dtype]) if rs is None else rs
+    assert np.array_equal(z[dropped], base[dropped]) and 0.13 < dropped.mean() < 0.17
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("B,N,L,D", [(2, 3, 150, 64), (1, 2, 70, 128), (1, 1, 300, 64)])
+def test_dropout_attention(K, gpu_device, dtype, B, N, L, D):
+    q, k, v = attn_inputs(B, N, L, D, dtype, gaussian=True, seed=21)
+    z = host(K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                                  dropout_prob=0.2))
+    want = O.flash_attention_v1(q, k, v, dropout_prob=0.2)
+    check_attention(z, want, v.astype(np.float32) / 0.8, dtype, "attention dropout")
+    # far from the p = 0 result, and the merged-heads layout carries the same values
+    assert np.abs(want.astype(np.float32) - O.flash_attention_v1(q, k, v).astype(np.float32)).max() > 0.05
+    zm = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                              dropout_prob=0.2, merged_heads_layout=True)
+    assert np.array_equal(host(zm), z)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_gpt2_train_mode_forward(gpu_device, dtype):
+    """model.train(): the dropout of GPTConfig reaches the embedding, the attention weights,
+    the attention projection and both ffn products (gpt.py:44-58, 92-109, 165-167)."""
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig
+
+    cfg = dict(n_layer=2, n_head=2, n_embd=128, vocab_size=211, block_size=96)
+    params = O.synthetic_params(**cfg, seed=5, std=0.05, dtype=NP[dtype])
+    ids = O.synthetic_ids(2, 80, cfg["vocab_size"], seed=5)
+    model = load_params(FusedGPT(GPTConfig(dropout=0.1, **cfg)), params, dtype, gpu_device)
+    model.train()
+    with torch.no_grad():
+        hidden = model(dev(ids, gpu_device))
+    want = O.gpt2_forward(params, ids, cfg["n_head"], dropout_prob=0.1)
+    eval_want = O.gpt2_forward(params, ids, cfg["n_head"])
+    assert np.abs(want.astype(np.float64) - eval_want).max() > 0.1  # the masks matter
+    if dtype == torch.float32:
+        check_model_fp32(host(hidden), want, "hidden (train mode)")
+    else:
+        assert np.abs(host(hidden).astype(np.float64) - want).max() <= 2e-2

@@ -53,7 +53,9 @@ def test_invalid_arguments_are_rejected_before_any_launch(lib):
     assert lib.gptmi_layernorm(fake, fake, fake, fake, 4, 10000, 1e-5, 1, None) == -2   # H too large
     assert b"8192" in lib.gptmi_last_error()
     assert lib.gptmi_embed(fake, fake, fake, fake, 1, 8, 4, 4, 8, 0.0, 0, 1, None) == -1  # L > P
-    assert lib.gptmi_embed(fake, fake, fake, fake, 1, 4, 4, 4, 8, 0.5, 0, 1, None) == -2  # dropout
+    assert lib.gptmi_embed(fake, fake, fake, fake, 1, 4, 4, 4, 8, 1.0, 0, 1, None) == -1  # p >= 1
+    assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 8, 64, 0.125, -0.1, 0, 0, 1,
+                                None) == -1                                             # p < 0
     assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 9, 64, 0.125, 0.0, 0, 0, 1,
                                 None) == -2                                             # Lq != Lk
     assert lib.gptmi_linear(fake, fake, None, None, fake, 4, 4, 4, 0, 0.0, 0, 0, None, 0, 1,
