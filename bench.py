@@ -3,6 +3,12 @@
 synthetic N(0, 0.02) weights and uniform token ids, one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload headline|batch2048|xl|ops] [--lm-head]
+
+The default (and the only line the contract asks for) is `headline`; `batch2048` is the same model
+at the max-batch memory point 2048 x 300, `xl` the GPT-2 XL shape (48 x 1600, 25 heads, batch 64 x
+seqlen 1024), `ops` times the single operators at the headline sizes (mean and median of
+event-timed repetitions, one JSON line).  `--lm-head` adds the tied LM head (logits) to the step.
 
 A step is one forward pass (hidden state [512, 300, 768], like the reference's forward, which
 stops at the final LayerNorm) with the token ids already resident in HBM.  Prints ONE JSON
@@ -26,21 +32,30 @@ if ROOT not in sys.path:
 
 BATCH, SEQLEN = 512, 300
 ARCH = dict(vocab_size=50257, block_size=1024, n_layer=12, n_head=12, n_embd=768)
+ARCH_XL = dict(vocab_size=50257, block_size=1024, n_layer=48, n_head=25, n_embd=1600)
+WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
+    "headline": (ARCH, 512, 300, "GPT-2 124M forward, fp16 storage / fp32 accumulate, batch 512 x "
+                                 "seqlen 300"),
+    "batch2048": (ARCH, 2048, 300, "GPT-2 124M forward, fp16 storage / fp32 accumulate, batch 2048 "
+                                   "x seqlen 300 (max-batch memory point)"),
+    "xl": (ARCH_XL, 64, 1024, "GPT-2 XL-shape forward (48 layers, d_model 1600, 25 heads x 64, FFN "
+                              "6400), fp16 storage / fp32 accumulate, batch 64 x seqlen 1024"),
+}
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
-FFN1 = dict(M=BATCH * SEQLEN, N=3072, K=768)
+PEAK_HBM = 8.0e12        # bytes/s
 # HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (890.7 MB after scaling by
 # the copy kernel of --traffic-calibration) + WRITE_SIZE (943.7 MB); the counters cannot be read
 # from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
 FFN1_TRAFFIC_BYTES = 1.834e9
 
 
-def forward_flops(tokens, seqlen):
-    """Executed FLOPs of one forward without LM head: the four GEMMs per layer plus the causal
-    half of the attention products."""
-    h, L = ARCH["n_embd"], ARCH["n_layer"]
+def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
+    """Executed FLOPs of one forward: the four GEMMs per layer plus the causal half of the
+    attention products (+ the tied LM head when asked for)."""
+    h, L = arch["n_embd"], arch["n_layer"]
     gemm = 2 * tokens * h * (3 * h + h + 4 * h + 4 * h)
-    attn = 4 * (tokens // seqlen) * ARCH["n_head"] * (h // ARCH["n_head"]) * seqlen * (seqlen + 1) // 2
-    return L * (gemm + attn)
+    attn = 4 * (tokens // seqlen) * arch["n_head"] * (h // arch["n_head"]) * seqlen * (seqlen + 1) // 2
+    return L * (gemm + attn) + (2 * tokens * h * arch["vocab_size"] if lm_head else 0)
 
 
 def cpu_baseline(sample_batch=16, reps=2):
@@ -88,11 +103,88 @@ def copy_calibration(dev, rows=262144, cols=2048, reps=3):
     assert torch.equal(dst.view(torch.float16).view(rows, cols), src)
 
 
+def time_op(fn, flush=None, min_ms=100.0, warm_ms=25.0):
+    """Mean and median duration (ms) of fn() from one event pair per repetition, after at
+    least warm_ms of warm-up and over at least min_ms of repetitions; `flush` (a callable) runs
+    before every repetition, outside the timed pair, to push the operands out of L2 / the
+    memory-side cache for the bandwidth-bound operators."""
+    import torch
+
+    def once():
+        if flush is not None:
+            flush()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        return e0, e1
+
+    e0, e1 = once()
+    torch.cuda.synchronize()
+    est = max(e0.elapsed_time(e1), 1e-3)
+    for _ in range(max(1, int(warm_ms / est))):
+        once()
+    pairs = [once() for _ in range(max(5, int(min_ms / est)))]
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in pairs)
+    return sum(ts) / len(ts), ts[len(ts) // 2], len(ts)
+
+
+def bench_ops(dev):
+    """Single operators at the headline sizes (M = 512 * 300 tokens)."""
+    import torch
+
+    from gpt_triton_amd import kernels as K
+
+    M, h = BATCH * SEQLEN, 768
+    g = torch.Generator(device=dev).manual_seed(1337)
+    rn = lambda *shape, std=1.0: (std * torch.randn(*shape, device=dev, generator=g)).half()
+    x, x4 = rn(M, h), rn(M, 4 * h)
+    w1, b1 = K.pack_weight(rn(h, 4 * h, std=0.02)), rn(4 * h, std=0.02)
+    w2, b2 = K.pack_weight(rn(4 * h, h, std=0.02)), rn(h, std=0.02)
+    wq, bq = K.pack_weight(rn(h, 3 * h, std=0.02)), rn(3 * h, std=0.02)
+    wo, bo = K.pack_weight(rn(h, h, std=0.02)), rn(h, std=0.02)
+    lw, lb = torch.ones(h, device=dev).half(), torch.zeros(h, device=dev).half()
+    q, k, v = (rn(BATCH, 12, SEQLEN, 64) for _ in range(3))
+    ids = torch.randint(0, ARCH["vocab_size"], (BATCH, SEQLEN), device=dev, generator=g)
+    wte, wpe = rn(ARCH["vocab_size"], h, std=0.02), rn(1024, h, std=0.02)
+    spill = torch.empty(1 << 29, dtype=torch.uint8, device=dev)  # 512 MB > L2 + memory-side cache
+    flush = lambda: spill.add_(1)
+    gemm = lambda n, k_: 2 * M * n * k_
+    ops = [
+        ("ffn1 768->3072 +bias+GELU", lambda: K.fused_ffn(x, w1, bias=b1, add_gelu=True), gemm(3072, 768), None, None),
+        ("ffn2 3072->768 +bias", lambda: K.fused_ffn(x4, w2, bias=b2), gemm(768, 3072), None, None),
+        ("ffn2 3072->768 +bias+residual", lambda: K.fused_ffn(x4, w2, bias=b2, residual=x), gemm(768, 3072), None, None),
+        ("qkv 768->2304 +bias, head-major split", lambda: K.matmul_and_split_qkv(x.view(BATCH, SEQLEN, h), wq, bq, 12), gemm(2304, 768), None, None),
+        ("attention projection 768->768 +bias+residual", lambda: K.fused_ffn(x, wo, bias=bo, residual=x), gemm(768, 768), None, None),
+        ("flash attention 512x12x300x64 causal", lambda: K.flash_attention_v1(q, k, v), 4 * BATCH * 12 * 64 * SEQLEN * (SEQLEN + 1) // 2, 4 * BATCH * 12 * SEQLEN * 64 * 2, flush),
+        ("layernorm 153600x768", lambda: K.fused_layer_norm(x, lw, lb), None, 2 * M * h * 2, flush),
+        ("softmax 153600x768", lambda: K.fused_softmax(x), None, 2 * M * h * 2, flush),
+        ("embedding 512x300x768", lambda: K.fused_embeddings(ids, wte, wpe), None, M * 8 + 2 * M * h * 2 + SEQLEN * h * 2, flush),
+    ]
+    rows = []
+    for name, fn, flops, nbytes, fl in ops:
+        mean, med, n = time_op(fn, fl)
+        row = {"op": name, "mean_ms": round(mean, 4), "median_ms": round(med, 4), "reps": n}
+        if flops:
+            row["tflops"] = round(flops / (mean * 1e-3) / 1e12, 1)
+            row["frac_mfma_peak"] = round(flops / (mean * 1e-3) / PEAK_FP16, 4)
+        if nbytes:
+            row["gbps"] = round(nbytes / (mean * 1e-3) / 1e9, 1)
+            row["frac_hbm_peak"] = round(nbytes / (mean * 1e-3) / PEAK_HBM, 4)
+        rows.append(row)
+    print(json.dumps({"metric": "operators_at_headline_sizes", "dtype": "f16", "data": "synthetic",
+                      "n_gpus": 1, "ops": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ops"], default="headline")
+    ap.add_argument("--lm-head", action="store_true",
+                    help="include the tied LM head (logits [T, 50257]) in the step")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the host-CPU leg (used under rocprofv3)")
     ap.add_argument("--traffic-calibration", action="store_true",
@@ -113,11 +205,15 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "ops":
+        return bench_ops(dev)
 
-    cfg = G.GPTConfig(dropout=0.1, **ARCH)
+    arch, batch, seqlen, what = WORKLOADS[args.workload]
+    headline = args.workload == "headline" and not args.lm_head
+    cfg = G.GPTConfig(dropout=0.1, **arch)
     model = G.FusedGPT(cfg).init_synthetic_(seed=1337).to(device=dev, dtype=torch.float16).eval()
     gen = torch.Generator(device="cpu").manual_seed(1338)
-    ids = torch.randint(0, ARCH["vocab_size"], (BATCH, SEQLEN), generator=gen).to(dev)
+    ids = torch.randint(0, arch["vocab_size"], (batch, seqlen), generator=gen).to(dev)
 
     # events around every ffn1 launch (the GELU GEMM) on the stream it is launched on
     ffn1_events = []
@@ -135,29 +231,31 @@ def main():
 
     recording = [False]
     G.fused_ffn = timed_ffn
+    step = (lambda: model(ids, return_logits=True)[0]) if args.lm_head else (lambda: model(ids))
 
     with torch.no_grad():
         for _ in range(args.warmup):
-            model(ids)
+            step()
         torch.cuda.synchronize()
         recording[0] = True
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            out = model(ids)
+            out = step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     recording[0] = False
-    assert out.shape == (BATCH, SEQLEN, ARCH["n_embd"]) and bool(torch.isfinite(out).all())
+    assert out.shape == (batch, seqlen, arch["n_embd"]) and bool(torch.isfinite(out).all())
 
     ms = dt / args.steps * 1e3
-    tokens = BATCH * SEQLEN
-    flops = forward_flops(tokens, SEQLEN)
+    tokens = batch * seqlen
+    flops = forward_flops(tokens, seqlen, arch, args.lm_head)
+    h = arch["n_embd"]
     ffn1_ms = sum(a.elapsed_time(b) for a, b in ffn1_events) / max(1, len(ffn1_events))
-    ffn1_flops = 2 * FFN1["M"] * FFN1["N"] * FFN1["K"]
+    ffn1_flops = 2 * tokens * 4 * h * h
     achieved = ffn1_flops / (ffn1_ms * 1e-3) / 1e12
 
     line = {
-        "metric": "gpt2_124m_forward_tokens_per_s",
+        "metric": "gpt2_124m_forward_tokens_per_s" if arch is ARCH else "gpt2_xl_forward_tokens_per_s",
         "baseline_metric": "GPT-2 124M fwd ms @512x300 fp16; tokens/s; MFU vs MI355X peak",
         "value": round(tokens / (ms * 1e-3), 1),
         "unit": "tokens/s",
@@ -167,25 +265,27 @@ def main():
         "ms_per_step": round(ms, 3),
         "higher_is_better": True,
         "scaling": "weak",
-        # the reference's published number for this forward is 273 ms on one A100-40GB
+        # the reference's published number for the headline forward is 273 ms on one A100-40GB
         # (README.md:17, bench.py:87-89); other hardware, so reported as a ratio of step times
-        "vs_baseline": round(273.0 / ms, 3),
+        "vs_baseline": round(273.0 / ms, 3) if headline else None,
         "vs_baseline_ref": "273 ms, gpt-triton mixed fp16, 1x A100 40GB (README.md:17)",
         "dtype": "f16",
         "data": "synthetic",
         "mfu": round(flops / (ms * 1e-3) / PEAK_FP16, 4),
         "mfu_flops": flops,
-        "mfu_note": "executed FLOPs without LM head (GEMMs + causal attention) / 2.5 PFLOP/s",
-        "config": {"workload": "GPT-2 124M forward, fp16 storage / fp32 accumulate, batch 512 x "
-                               "seqlen 300, hidden-state output (no LM head)",
-                   "tokens_per_step": tokens, "n_layer": 12, "n_embd": 768, "n_head": 12},
-        "roofline": {"kernel": "gemm_kernel (ffn1: M=153600 N=3072 K=768, bias+GELU epilogue)",
+        "mfu_note": ("executed FLOPs with the tied LM head" if args.lm_head else
+                     "executed FLOPs without LM head") + " (GEMMs + causal attention) / 2.5 PFLOP/s",
+        "config": {"workload": what + (", logits output (tied LM head)" if args.lm_head
+                                       else ", hidden-state output (no LM head)"),
+                   "tokens_per_step": tokens, "n_layer": arch["n_layer"], "n_embd": h,
+                   "n_head": arch["n_head"]},
+        "roofline": {"kernel": f"gemm_kernel (ffn1: M={tokens} N={4 * h} K={h}, bias+GELU epilogue)",
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16 / 1e12,
                      "unit": "TFLOP/s", "frac": round(achieved * 1e12 / PEAK_FP16, 4),
                      "avg_ms": round(ffn1_ms, 4), "launches": len(ffn1_events),
-                     "traffic": FFN1_TRAFFIC_BYTES},
+                     "traffic": FFN1_TRAFFIC_BYTES if arch is ARCH and batch == BATCH else None},
     }
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
+    line["cpu_baseline"] = None if (args.no_cpu_baseline or not headline) else cpu_baseline()
     if args.traffic_calibration:
         copy_calibration(dev)
     print(json.dumps(line), flush=True)

@@ -303,6 +303,19 @@ def test_flash_attention_merged_heads_layout(K, gpu_device, dtype):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("D", [16, 32])
+def test_flash_attention_small_heads(K, gpu_device, dtype, D):
+    """Head sizes 16 and 32 (accepted by the reference, kernels.py:490) run zero padded to 64."""
+    q, k, v = attn_inputs(2, 3, 130, D, dtype, gaussian=True, seed=9)
+    z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+    assert z.shape == (2, 3, 130, D) and z.is_contiguous()
+    check_attention(host(z), O.flash_attention_v1(q, k, v), v, dtype, f"d={D}")
+    zm = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                              merged_heads_layout=True)
+    assert np.array_equal(host(zm), host(z))
+
+
 def test_flash_attention_xl_sequence(K, gpu_device):
     """BASELINE config 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
     K/V do not fit the resident variant)."""
