@@ -306,17 +306,19 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
 // Resident-K/V variant for short sequences (L*D small enough that K and V^T of
 // one (batch, head) fit in half a CU's LDS, e.g. L <= 320 at D = 64).
 //
-// One workgroup = 4 wavefronts = one (batch, head).  K ([L][D], 16-byte chunks
+// One workgroup = 8 wavefronts (4 for head sizes above 64, which need more than 128
+// registers) = one (batch, head).  K ([L][D], 16-byte chunks
 // swizzled with (row >> 1) & 7) and V^T ([D][Lp + 4], Lp = L rounded up to 64;
 // the 8 pad bytes per row spread the 32 rows a fragment read touches over all
 // banks) are staged once, behind ONE barrier; after it the wavefronts never
 // synchronise again.  Queries are cut into chunks of 32; chunk c costs
-// c/2 + 1 key tiles (causal), and the chunks are dealt to the 4 wavefronts in
-// snake order from the most expensive one, which balances the triangle (L = 300:
-// 8, 8, 7, 7 tiles).  The arithmetic per tile is that of the tiled kernel.
+// c/2 + 1 key tiles (causal), and the chunks are dealt to the wavefronts in snake
+// order from the most expensive one, which balances the triangle over the SIMDs
+// (L = 300: 8, 8, 7, 7 tiles).  The arithmetic per tile is that of the tiled kernel.
+// GPTMI_ATTN_NO_STAGE / GPTMI_ATTN_NO_COMPUTE are ablation switches of tuning builds.
 // ---------------------------------------------------------------------------
-template <int D, typename T, bool BLND>
-__global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
+template <int D, typename T, bool BLND, int NW>
+__global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     T* __restrict__ O, int heads, int L, float scale) {
   constexpr int CH = D / 8, KS = D / 16, DB = D / 32;
@@ -333,40 +335,56 @@ __global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
   const T* Kp = K + base;
   const T* Vp = V + base;
 
-  // ---- stage K: chunk s -> row s / CH, chunk s % CH --------------------------
-  for (int s0 = 0; s0 < L * CH; s0 += 256 * 4) {
-    h8 r[4];
+  // ---- stage K and V^T: every global load is requested before the first LDS store, so the
+  // workgroup pays one memory round trip, not one per batch.  The 80 KB limit bounds the
+  // work: at most 2560 16-byte chunks of K and 640 (4 keys x 8 d) units of V.
+  //   K chunk s -> row s / CH, chunk s % CH
+  //   V unit  u -> d-chunk u % CH, key group u / CH (4 keys); keys past the end repeat the
+  //   last row: their weights are exactly 0
+  constexpr int NT = NW * 64;
+  constexpr int KI = 2560 / NT, VI = (640 + NT - 1) / NT;
+  const int kchunks = L * CH, units = (Lp / 4) * CH;
+  h8 kr[KI], vr[VI][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int s = s0 + i * 256 + tid;
-      if (s < L * CH) r[i] = Ld8<T>::load(Kp + (int64_t)(s / CH) * D + (s % CH) * 8);
-    }
+  for (int i = 0; i < KI; ++i) {
+    const int s = i * NT + tid;
+#ifdef GPTMI_ATTN_NO_STAGE
+    kr[i] = zero_h8();
+#else
+    if (s < kchunks) kr[i] = Ld8<T>::load(Kp + (int64_t)(s / CH) * D + (s % CH) * 8);
+#endif
+  }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int s = s0 + i * 256 + tid;
-      if (s < L * CH) {
-        const int row = s / CH, c = s % CH;
-        *reinterpret_cast<h8*>(ks_ + row * (D * 2) + ((c ^ ((row >> 1) & 7)) << 4)) = r[i];
-      }
+  for (int i = 0; i < VI; ++i) {
+    const int u = i * NT + tid;
+    const int c = u % CH, kg = u / CH;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      int key = kg * 4 + kk;
+      key = key < L ? key : L - 1;
+#ifdef GPTMI_ATTN_NO_STAGE
+      vr[i][kk] = zero_h8();
+#else
+      if (u < units) vr[i][kk] = Ld8<T>::load(Vp + (int64_t)key * D + c * 8);
+#endif
     }
   }
-  // ---- stage V^T: unit u -> d-chunk u % CH, key group u / CH (4 keys) ---------
-  // keys past the end repeat the last row: their weights are exactly 0
-  const int units = (Lp / 4) * CH;
-  for (int u0 = 0; u0 < units; u0 += 256) {
-    const int u = u0 + tid;
+#pragma unroll
+  for (int i = 0; i < KI; ++i) {
+    const int s = i * NT + tid;
+    if (s < kchunks) {
+      const int row = s / CH, c = s % CH;
+      *reinterpret_cast<h8*>(ks_ + row * (D * 2) + ((c ^ ((row >> 1) & 7)) << 4)) = kr[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VI; ++i) {
+    const int u = i * NT + tid;
     if (u < units) {
       const int c = u % CH, kg = u / CH;
-      h8 r[4];
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        int key = kg * 4 + kk;
-        key = key < L ? key : L - 1;
-        r[kk] = Ld8<T>::load(Vp + (int64_t)key * D + c * 8);
-      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        h4 col = {r[0][j], r[1][j], r[2][j], r[3][j]};
+        h4 col = {vr[i][0][j], vr[i][1][j], vr[i][2][j], vr[i][3][j]};
         *reinterpret_cast<h4*>(vs_ + (c * 8 + j) * vstride + kg * 8) = col;
       }
     }
@@ -375,11 +393,12 @@ __global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
 
   const int ql = lane & 31, g = lane >> 5;
   const int nc = (L + 31) / 32;
-  // snake deal: position i (chunk nc-1-i) goes to wavefront i%8 < 4 ? i%8 : 7 - i%8
-  for (int i0 = 0; i0 < nc; i0 += 8) {
+  // snake deal over NW wavefronts: of every 2*NW positions (position i = chunk nc-1-i,
+  // most expensive first) wavefront w takes w and 2*NW-1-w
+  for (int i0 = 0; i0 < nc; i0 += 2 * NW) {
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      const int i = i0 + (half == 0 ? wave : 7 - wave);
+      const int i = i0 + (half == 0 ? wave : 2 * NW - 1 - wave);
       if (i >= nc) continue;
       const int qw0 = (nc - 1 - i) * 32;  // first query of the chunk
       const int q = qw0 + ql;
@@ -395,7 +414,11 @@ __global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
       float mrun = -INFINITY, den = 0.f;
       int last_q = qw0 + 31;
       if (last_q > L - 1) last_q = L - 1;
+#ifdef GPTMI_ATTN_NO_COMPUTE
+      const int nt = L > (1 << 30) ? 1 : 0;
+#else
       const int nt = last_q / BKEY + 1;
+#endif
       for (int t = 0; t < nt; ++t) {
         const int k0 = t * BKEY;
         // ---- S^T = K . Q^T -----------------------------------------------------
@@ -528,6 +551,11 @@ __global__ __launch_bounds__(256, 2) void flash_attn_resident_kernel(
   }
 }
 
+#ifndef GPTMI_RESIDENT_WAVES
+#define GPTMI_RESIDENT_WAVES 8
+#endif
+constexpr int RESIDENT_WAVES = GPTMI_RESIDENT_WAVES;
+
 // LDS bytes of the resident variant, or 0 if this (L, D) does not fit two workgroups per CU.
 inline size_t resident_lds_bytes(int L, int D) {
   const int Lp = (L + BKEY - 1) / BKEY * BKEY;
@@ -538,7 +566,8 @@ inline size_t resident_lds_bytes(int L, int D) {
 template <int D, typename T, bool BLND>
 int launch_resident(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
                     int L, float scale, size_t lds, hipStream_t st) {
-  auto kern = flash_attn_resident_kernel<D, T, BLND>;
+  constexpr int NW = D == 64 ? RESIDENT_WAVES : 4;  // larger heads need > 128 registers
+  auto kern = flash_attn_resident_kernel<D, T, BLND, NW>;
   static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -549,7 +578,7 @@ int launch_resident(const void* q, const void* k, const void* v, void* out, int6
     }
     attr_done = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)BN), dim3(256), lds, st, (const T*)q, (const T*)k,
+  hipLaunchKernelGGL(kern, dim3((unsigned)BN), dim3(NW * 64), lds, st, (const T*)q, (const T*)k,
                      (const T*)v, (T*)out, heads, L, scale);
   return 0;
 }
