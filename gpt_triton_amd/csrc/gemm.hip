@@ -378,6 +378,13 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       lds_dma16(b_src[it] + (size_t)kt * ROWB, bs + it * T_ * 16);
   };
 
+  // one of the A_IT + B_IT loads of k-tile kt (the A loads come first)
+  auto issue_one = [&](int kt, int n) {
+    const unsigned as = wave_off + (kt % NST) * STAGE;
+    if (n < A_IT) lds_dma16(a_src[n] + (size_t)kt * ROWB, as + n * T_ * 16);
+    else lds_dma16(b_src[n - A_IT] + (size_t)kt * ROWB, as + BM * ROWB + (n - A_IT) * T_ * 16);
+  };
+
   f16v acc[NB][MB];
 #pragma unroll
   for (int i = 0; i < NB; ++i)
@@ -410,86 +417,82 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
             __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j], 0, 0, 0);
   };
 
+  // The MFMAs of one k-slice with the loads of k-tile kt_load dealt between them: a load
+  // instruction (address add, M0, issue) then costs no MFMA time -- issued as one block right
+  // behind the barrier, the loads of all wavefronts kept the matrix pipe idle for ~500 cycles
+  // per k-tile.
+  auto mma_and_issue = [&](int slot, int kt_load, bool go) {
+    constexpr int PER = (A_IT + B_IT + MB * NB - 1) / (MB * NB);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < MB; ++j) {
+        acc[i][j] =
+            __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int l = 0; l < PER; ++l) {
+          const int n = (i * MB + j) * PER + l;  // a constant after unrolling
+          if (n < A_IT + B_IT && go) issue_one(kt_load, n);
+        }
+      }
+  };
+
   const int KT = Kp / BKS;
 #ifdef GPTMI_NO_LOADS
   constexpr bool loads = false;
 #else
   constexpr bool loads = true;
 #endif
+  // Pipeline.  NST k-tiles are in LDS or on their way at any time.  Fragments of the next
+  // k-slice are requested before the MFMAs of the current one issue (the scheduling fences keep
+  // the compiler from sinking the reads behind the MFMAs again).  In front of the LAST k-slice of
+  // tile kt -- whose fragments are in registers by then -- tile kt+1 is published (own loads
+  // landed, own LDS reads retired, barrier), its first fragments are requested, and the stage of
+  // tile kt, which nobody reads any more, is refilled with tile kt+NST while that last slice is
+  // multiplied.  No MFMA ever waits for a barrier plus an LDS round trip.
   if (loads) {
 #pragma unroll
-    for (int s = 0; s < NST - 1; ++s)
+    for (int s = 0; s < NST; ++s)
       if (s < KT) issue(s);
-    // tile 0 must have landed; up to NST-2 younger tiles stay in flight
-    if (KT >= NST - 1) wait_vmcnt<(NST - 2) * LPT>();
+    // tile 0 must have landed; up to NST-1 younger tiles stay in flight
+    if (KT >= NST) wait_vmcnt<(NST - 1) * LPT>();
     else wait_vmcnt<0>();
   }
   asm volatile("s_barrier" ::: "memory");
-  if constexpr (NST > 2) read_frags(0, 0, 0);
+  read_frags(0, 0, 0);
 #ifdef GPTMI_TUNING
   const unsigned long long t_pro = __builtin_amdgcn_s_memtime();
 #endif
 
-  if constexpr (NST == 2) {
-    // Plain double buffering (the only depth a 256x256x64 stage leaves room for): tile kt+1
-    // streams in while tile kt is multiplied; one barrier per tile.
-    for (int kt = 0; kt < KT; ++kt) {
-      if (kt > 0) {
-        if (loads) wait_vmcnt<0>();
-        block_barrier();
-      }
-      if (kt + 1 < KT && loads) issue(kt + 1);
-      read_frags(kt, 0, 0);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int cur = ks & 1;
-        if (ks + 1 < KS) read_frags(kt, ks + 1, cur ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-#ifndef GPTMI_NO_MFMA
-        mma(cur);
-#else
-#pragma unroll
-        for (int j = 0; j < MB; ++j) acc[0][j][0] += (float)af[cur][j][0] + (float)af[cur][j][7];
-#pragma unroll
-        for (int i = 0; i < NB; ++i) acc[i][0][1] += (float)bf[cur][i][0] + (float)bf[cur][i][7];
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  } else {
-  // Fragments of the next k-step are requested before the MFMAs of this one
-  // issue; the scheduling fences keep the compiler from sinking the reads
-  // behind the MFMAs again.  In front of the last k-step of a tile the next
-  // tile is published (own loads landed, then the barrier) and the ring slot
-  // of tile kt-1, which every wavefront has finished reading, is refilled.
   for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int cur = ks & 1;
-      if (ks + 1 < KS) {
+      const bool last = ks + 1 == KS;
+      if (!last) {
         read_frags(kt, ks + 1, cur ^ 1);
-      } else {
-        if (kt + 1 < KT && loads) {
-          // tile kt+1 complete; tiles kt+2 .. kt+NST-2 may still be in flight
-          if (kt + NST - 2 < KT) wait_vmcnt<(NST > 2 ? (NST - 3) * LPT : 0)>();
+      } else if (kt + 1 < KT) {
+        if (loads) {
+          // tile kt+1 complete; tiles kt+2 .. kt+NST-1 may still be in flight
+          if (kt + NST - 1 < KT) wait_vmcnt<(NST - 2) * LPT>();
           else wait_vmcnt<0>();
         }
-        asm volatile("s_barrier" ::: "memory");
-        if (kt + NST - 1 < KT && loads) issue(kt + NST - 1);
-        read_frags(kt + 1, 0, cur ^ 1);  // past the last tile this reads a dead stage
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        read_frags(kt + 1, 0, cur ^ 1);
       }
       __builtin_amdgcn_sched_barrier(0);
 #ifndef GPTMI_NO_MFMA
-      mma(cur);
+      if (last) mma_and_issue(cur, kt + NST, kt + NST < KT && loads);
+      else mma(cur);
 #else
 #pragma unroll
       for (int j = 0; j < MB; ++j) acc[0][j][0] += (float)af[cur][j][0] + (float)af[cur][j][7];
 #pragma unroll
       for (int i = 0; i < NB; ++i) acc[i][0][1] += (float)bf[cur][i][0] + (float)bf[cur][i][7];
+      if (last && kt + NST < KT && loads) issue(kt + NST);
 #endif
       __builtin_amdgcn_sched_barrier(0);
     }
-  }
   }
 
   // ---- epilogue -----------------------------------------------------------
