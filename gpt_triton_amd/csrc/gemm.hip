@@ -334,6 +334,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   const int wm = wave % WM, wn = wave / WM;
 #ifdef GPTMI_TUNING
   const unsigned long long t_start = __builtin_amdgcn_s_memtime();
+  const unsigned long long r_start = __builtin_amdgcn_s_memrealtime();
 #endif
   // Tile order: the column tiles are cut into groups of group_w; inside a group the column
   // runs fastest, then the row block, and the groups follow each other.  Workgroups that run
@@ -518,16 +519,15 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #endif
 #ifdef GPTMI_TUNING
   if (ep.trace && tid == 0) {
-    unsigned hw, xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    // shader-clock stamps of the phases, and the constant 100 MHz clock around the whole
+    // workgroup (the ratio of the two spans is the shader clock the workgroup ran at)
     unsigned long long* t = ep.trace + (size_t)blockIdx.x * 6;
     t[0] = t_start;
     t[1] = t_pro;
     t[2] = t_loop;
     t[3] = __builtin_amdgcn_s_memtime();
-    t[4] = hw;
-    t[5] = xcc;
+    t[4] = r_start;
+    t[5] = __builtin_amdgcn_s_memrealtime();
   }
 #endif
 }
