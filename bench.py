@@ -194,7 +194,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's full share of the forward; "
-                 "--gpus must be 1 (the path shards over the batch with no exchange, see DESIGN.md)")
+                 "--gpus must be 1 (the forward shards over the batch with no exchange between GPUs)")
 
     import torch
 

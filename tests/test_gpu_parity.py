@@ -4,7 +4,7 @@ the GPT-2 sizes; the full BASELINE sizes are checked on sub-samples of independe
 
 Tolerances (stated once, used everywhere):
   * embedding gather: bit exact;
-  * fp32 storage: |a-b| <= 1e-4 * |b| + 1e-4 * max|b| elementwise (north-star "fp32 outputs
+  * fp32 storage: |a-b| <= 1e-4 * |b| + 1e-4 * max|b| elementwise (the target "fp32 outputs
     within 1e-4 relative"; the reference itself only uses torch.allclose with an absolute
     tolerance, test.py:44,59,87,117).  The strict max|a-b| / max|b| is printed on failure.
     Attention in fp32 storage is the one exception (check_attention): fp32 sums inside the
@@ -404,7 +404,7 @@ def test_gpt2_124m_config0(gpu_device, dtype):
 def test_gpt2_layerwise_fp32(K, gpu_device):
     """Every operator of a 3-layer model, each fed the ORACLE's intermediate activations, so
     that no upstream difference is carried along: fp32 storage, tolerance 1e-5 * max|b| (the
-    north-star asks for 1e-4), attention through check_attention."""
+    target for this build is 1e-4), attention through check_attention."""
     cfg = dict(n_layer=3, n_head=4, n_embd=256, vocab_size=1000, block_size=128)
     P = O.synthetic_params(**cfg, seed=3, std=0.05, dtype=np.float32)
     ids = O.synthetic_ids(3, 100, cfg["vocab_size"], seed=3)
