@@ -610,3 +610,70 @@ def test_gpt2_train_mode_forward(gpu_device, dtype):
         check_model_fp32(host(hidden), want, "hidden (train mode)")
     else:
         assert np.abs(host(hidden).astype(np.float64) - want).max() <= 2e-2
+
+
+# ----------------------------------------------------------------------------- numerical edges
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_layer_norm_large_mean_small_spread(K, gpu_device, dtype):
+    """Rows with mean 1000 and spread 1: only the centred (two-pass) variance of the reference
+    (kernels.py:123-129) survives this; E[x^2] - E[x]^2 in fp32 loses every digit.  Also
+    constant rows (variance 0 -> output = bias)."""
+    r = np.random.default_rng(3)
+    x = (1000 + r.standard_normal((37, 768))).astype(NP[dtype])
+    x[5] = 1024  # sums of a power of two are exact: the centred row is exactly 0
+    w = (1 + 0.1 * r.standard_normal(768)).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(768)).astype(NP[dtype])
+    z = host(K.fused_layer_norm(dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device)))
+    want = O.fused_layer_norm(x, w, b)
+    check(z, want, dtype, "layer norm, mean 1000")
+    assert np.array_equal(z[5], b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_softmax_extreme_values(K, gpu_device, dtype):
+    r = np.random.default_rng(4)
+    x = np.clip(r.standard_normal((9, 500)) * 20000, -60000, 60000).astype(NP[dtype])
+    x[0] = 0
+    x[1, 3] = -np.inf
+    z = host(K.fused_softmax(dev(x, gpu_device)))
+    want = O.softmax_rows(x)
+    check(z, want, dtype, "softmax, huge logits")
+    assert z[1, 3] == 0 and np.allclose(z.astype(np.float64).sum(-1), 1, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_gelu_epilogue_saturates_without_nan(K, gpu_device, dtype):
+    """|z| up to 6e4 in front of the GELU: exp2 overflows to inf on the negative side and the
+    result must be -0 / z, never NaN (the reference's tanh form saturates, kernels.py:15-26)."""
+    x = np.zeros((64, 64), NP[dtype])
+    x[:, 0] = 1
+    w = np.zeros((64, 128), NP[dtype])
+    w[0] = np.linspace(-60000, 60000, 128).astype(NP[dtype])
+    z = host(K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), add_gelu=True))
+    want = O.fused_ffn(x, w, add_gelu=True)
+    assert np.isfinite(z).all()
+    check(z, want, dtype, "gelu saturation")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_attention_large_scores(K, gpu_device, dtype):
+    """Scores of a few hundred: all but a handful of weights underflow, the running max moves
+    by hundreds between tiles."""
+    r = np.random.default_rng(6)
+    q, k, v = (r.standard_normal((1, 2, 200, 64)).astype(NP[dtype]) for _ in range(3))
+    q *= 12
+    k *= 12
+    z = host(K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device)))
+    assert np.isfinite(z).all()
+    check_attention(z, O.flash_attention_v1(q, k, v), v, dtype, "attention, large scores")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd", [(1, 1, 1), (1, 257, 65), (3, 8, 4096)])
+def test_fused_ffn_degenerate_sizes(K, gpu_device, dtype, M, N, Kd):
+    r = np.random.default_rng(8)
+    x = r.standard_normal((M, Kd)).astype(NP[dtype])
+    w = (r.standard_normal((Kd, N)) / math.sqrt(Kd)).astype(NP[dtype])
+    b = r.standard_normal(N).astype(NP[dtype])
+    z = host(K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device)))
+    check(z, O.fused_ffn(x, w, bias=b), dtype, f"ffn {M}x{N}x{Kd}")
