@@ -69,6 +69,32 @@ __device__ __forceinline__ void lds_dma16(const void* gsrc, unsigned lds_off) {
                : "memory", "m0");
 }
 
+// The same with a wavefront-uniform 64-bit base in scalar registers and a 32-bit per-lane
+// byte offset: one VGPR per load instead of an address pair, and the k-step is a scalar add.
+__device__ __forceinline__ void lds_dma16_base(const void* base, unsigned lane_off,
+                                               unsigned lds_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_off), "v"(lane_off), "s"(base)
+               : "memory", "m0");
+}
+
+// Streaming store of 4 output elements at (wavefront-uniform 64-bit base) + (32-bit lane
+// offset).  Written as assembly because the compiler otherwise materialises one 64-bit address
+// pair per store of an unrolled epilogue and spills.
+__device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, h4 v) {
+  asm volatile("global_store_dwordx2 %0, %1, %2 nt" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
+}
+__device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, f4 v) {
+  // a store of more than 64 bits reads its data registers a little after issue: the wait states
+  // keep the next VALU instruction from overwriting them (the compiler adds these for its own
+  // stores, it cannot for assembly)
+  asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
+               :
+               : "v"(lane_off), "v"(v), "s"(base)
+               : "memory");
+}
+
 // Workgroup barrier that does not drain the vector-memory counter: the
 // compiler's own barrier waits for vmcnt(0), which would serialise the
 // global->LDS prefetch of the younger pipeline stages behind it.
@@ -575,6 +601,319 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// Streaming variant of the 256x256x64 kernel: one workgroup per CU walks tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ...  The two operand stages keep alternating across tile
+// boundaries, so the first two k-tiles of the NEXT output tile are requested while the current
+// one finishes, and the epilogue runs with those loads in flight.  What this removes, per tile
+// of ~28 us: the pipeline fill (3.5 k cycles) and the ~2.8 us a CU otherwise sits idle between
+// two workgroups while the stores of the one that ended drain (measured: 231 of 256 CUs busy
+// on average with one workgroup per tile, 251 when the kernel stores nothing).
+//
+// LDS: stages at [0, 128 KB), epilogue slabs behind them (8 wavefronts x 4 KB: one 32 x 32 fp32
+// block, 16-byte units XOR-swizzled with (row >> 1) & 7), so the epilogue never touches a stage.
+//
+// Load/store counter.  Loads and stores of a wavefront retire in issue order on this ISA.  The
+// loads of the next tile's k-tile 1 are issued BEFORE the epilogue's stores, so waiting for them
+// with vmcnt(16) -- 32 younger stores exist after the epilogue -- does not wait for the stores'
+// acknowledgements.  The bias is fetched, and waited for, before those loads are issued, so
+// that no compiler-placed wait inside the epilogue falls behind them.  Only whole tiles, no
+// residual, no dropout: the launcher sends everything else to gemm_kernel.
+// ---------------------------------------------------------------------------
+template <int MB, int NB, typename T, bool QKV, bool GELU>
+__device__ __forceinline__ void store_wave_tile32(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+                                                  const EpiDev& ep, int64_t mw0, int nw0, int N,
+                                                  char* slab, int lane) {
+  typedef typename Pack4<T>::type P4;
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int rrow = lane >> 3, runit = lane & 7;
+  T* qkv_col[NB];
+  unsigned b0 = 0, l0 = 0;
+  const unsigned Lu = (unsigned)ep.L;
+  const bool step_rows = Lu >= 32u * MB;
+  if (QKV) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) qkv_col[i] = qkv_column_base<T>(ep, nw0 + i * 32 + runit * 4);
+    const unsigned m_first = (unsigned)mw0 + (unsigned)rrow;
+    b0 = m_first / Lu;
+    l0 = m_first - b0 * Lu;
+  }
+  const int64_t batch_stride = (int64_t)ep.heads * ep.L * ep.d;
+  // byte offset of this lane's (row, 4 columns) inside a 32 x 32 pass of a row-major [.][N] matrix
+  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 4) * (unsigned)sizeof(T);
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f4 z;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          z[e] = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          if (GELU) z[e] = gelu_new(z[e]);
+        }
+        *reinterpret_cast<f4*>(slab + frow * 128 + (((g * 2 + fhalf) ^ fkey) << 4)) = z;
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int row = rr * 8 + rrow;
+        const f4 z =
+            *reinterpret_cast<const f4*>(slab + row * 128 + ((runit ^ ((row >> 1) & 7)) << 4));
+        P4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (T)z[e];
+        if constexpr (QKV) {
+          unsigned b, l;
+          if (step_rows) {
+            b = b0;
+            l = l0 + (unsigned)(j * 32 + rr * 8);
+            if (l >= Lu) { l -= Lu; ++b; }
+          } else {
+            const unsigned m = (unsigned)mw0 + (unsigned)(j * 32 + row);
+            b = m / Lu;
+            l = m - b * Lu;
+          }
+          T* dst = qkv_col[i] + ((int64_t)b * batch_stride + (int64_t)l * ep.d);
+          __builtin_nontemporal_store(o, reinterpret_cast<P4*>(dst));
+        } else {
+          // wavefront-uniform 64-bit part in scalar registers + one 32-bit lane offset
+          store_nt_base(reinterpret_cast<char*>(ep.out) +
+                            ((mw0 + j * 32 + rr * 8) * (int64_t)N + (nw0 + i * 32)) *
+                                (int64_t)sizeof(T),
+                        lane_byte_off, o);
+        }
+      }
+    }
+  }
+}
+
+template <int WM, int WN, typename T, bool QKV>
+__global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
+    const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
+    int tiles_m, int tiles_n, int group_w, EpiDev ep) {
+  constexpr int BM = 256, BN = 256, ROWB = 128, T_ = 512, KS = 4;
+  static_assert(WM * WN == 8, "8 wavefronts");
+  constexpr int TM = BM / WM, TN = BN / WN;
+  constexpr int MB = TM / 32, NB = TN / 32;
+  constexpr int A_IT = 4, B_IT = 4, LPT = A_IT + B_IT;  // 16-byte loads per thread per k-tile
+  constexpr int STAGE = (BM + BN) * ROWB;               // 64 KB
+  constexpr int SLABS = 2 * STAGE;                      // epilogue slabs start behind the stages
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  // provably wavefront-uniform, so that everything derived from the wavefront's sub-tile origin
+  // (output and residual bases) lives in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  const int num_tiles = tiles_m * tiles_n;
+  const int KT = Kp / 64;  // >= 2 (checked by the launcher)
+
+  // Operand-tile slot s = it * 512 + tid: row it * 64 + tid / 8, 16-byte position tid % 8,
+  // which holds source chunk (tid % 8) ^ ((row >> 1) & 7) -- the key does not depend on `it`.
+  // M and N are multiples of 256 here (the launcher sends other shapes to gemm_kernel), so no
+  // row is clamped: a load address is a per-tile scalar base (first row of the tile, k-tile
+  // offset) plus one of four per-thread 32-bit offsets shared by A and B.
+  const int r0 = tid >> 3;
+  unsigned lane_off[A_IT];
+#pragma unroll
+  for (int it = 0; it < A_IT; ++it)
+    lane_off[it] = (unsigned)(r0 + it * 64) * (unsigned)Kp * 2u +
+                   (unsigned)(((tid & 7) ^ ((r0 >> 1) & 7)) * 16);
+  const unsigned wave_off =
+      __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + (unsigned)wave * 1024u);
+  auto tile_origin = [&](int vp, int& m0, int& n0) {
+    const int tile = xcd_tile(vp, num_tiles);
+    const int grp = tile / (tiles_m * group_w);
+    const int in_grp = tile - grp * tiles_m * group_w;
+    const int grp_w = min(group_w, tiles_n - grp * group_w);
+    m0 = (in_grp / grp_w) * BM;
+    n0 = (grp * group_w + in_grp % grp_w) * BN;
+  };
+  // load n (0..3: A, 4..7: B) of k-tile k of the tile at (m0, n0) into `stage`
+  auto issue_one = [&](int stage, int m0, int n0, int k, int n) {
+    const unsigned base = wave_off + stage * STAGE;
+    if (n < A_IT)
+      lds_dma16_base((const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB), lane_off[n],
+                     base + n * T_ * 16);
+    else
+      lds_dma16_base((const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB),
+                     lane_off[n - A_IT], base + BM * ROWB + (n - A_IT) * T_ * 16);
+  };
+  auto issue = [&](int stage, int m0, int n0, int k) {
+#pragma unroll
+    for (int n = 0; n < LPT; ++n) issue_one(stage, m0, n0, k, n);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int a_row_off = (wm * TM + frow) * ROWB;
+  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
+  h8 af[2][MB], bf[2][NB];
+  auto read_frags = [&](int stage, int ks, int slot) {
+    const char* st = smem + stage * STAGE;
+    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
+#pragma unroll
+    for (int j = 0; j < MB; ++j)
+      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
+  };
+
+  int vp = blockIdx.x;
+  int m0, n0;
+  tile_origin(vp, m0, n0);
+  issue(0, m0, n0, 0);
+  issue(1, m0, n0, 1);
+  wait_vmcnt<LPT>();
+  asm volatile("s_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+  int stage = 0;           // stage of the k-tile being multiplied
+  bool first_tile = true;
+
+  while (true) {
+    const int vp_next = vp + (int)gridDim.x;
+    const bool has_next = vp_next < num_tiles;
+    int m0_n = 0, n0_n = 0;
+    if (has_next) tile_origin(vp_next, m0_n, n0_n);
+    const int64_t mw0 = (int64_t)m0 + wm * TM;
+    const int nw0 = n0 + wn * TN;
+
+    f16v acc[NB][MB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < MB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    auto mma = [&](int slot) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
+                                                             0, 0, 0);
+    };
+    // k-slices 0..2 of the k-tile in `stage`: fragments of the next slice first, then the MFMAs
+    auto first_slices = [&]() {
+#pragma unroll
+      for (int ks = 0; ks < KS - 1; ++ks) {
+        read_frags(stage, ks + 1, (ks & 1) ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(ks & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // publish the k-tile in the other stage and fetch its first fragments (slot 0)
+    auto publish_next = [&](bool behind_epilogue, bool fetch) {
+      if (behind_epilogue) wait_vmcnt<16>();
+      else wait_vmcnt<0>();
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (fetch) read_frags(stage ^ 1, 0, 0);
+    };
+
+    // all k-tiles but the last: the final slice refills this stage with the k-tile two ahead
+    // (of this tile, or the first of the next one), the loads dealt between the MFMAs
+    for (int kt = 0; kt + 1 < KT; ++kt) {
+      first_slices();
+      publish_next(kt == 0 && !first_tile, true);
+      const bool own = kt + 2 < KT;
+      const bool go = own || has_next;
+      const int ra = own ? m0 : m0_n, rb = own ? n0 : n0_n;
+      const int kk = own ? kt + 2 : 0;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
+          if (go) issue_one(stage, ra, rb, kk, i * MB + j);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+      stage ^= 1;
+    }
+
+    // last k-tile: before its final slice the next tile's first k-tile is published (this
+    // stage is free for a refill then); the bias is fetched and waited for BEFORE the next
+    // tile's second k-tile is requested, so that no wait inside the epilogue falls behind those
+    // loads.  The next tile's first fragments are read after the epilogue (registers).
+    first_slices();
+    if (has_next) publish_next(false, false);
+    f4 bias_r[NB][4];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
+        f4 b = {0.f, 0.f, 0.f, 0.f};
+        if (ep.bias) {
+          const typename Pack4<T>::type t =
+              *reinterpret_cast<const typename Pack4<T>::type*>((const T*)ep.bias + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
+        }
+        bias_r[i][g] = b;
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
+    if (has_next) issue(stage, m0_n, n0_n, 1);
+    stage ^= 1;
+
+    // ---- epilogue: the next tile's first two k-tiles are landing meanwhile ----
+    {
+      char* slab = smem + SLABS + wave * 4096;
+      if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+      else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+    }
+    if (!has_next) break;
+    read_frags(stage, 0, 0);
+    first_tile = false;
+    vp = vp_next;
+    m0 = m0_n;
+    n0 = n0_n;
+  }
+}
+
+template <int WM, int WN, typename T, bool QKV>
+int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+                  hipStream_t st) {
+  auto kern = gemm_stream_kernel<WM, WN, T, QKV>;
+  constexpr int smem = 2 * 512 * 128 + 8 * 4096;  // 160 KB: two stages + the epilogue slabs
+  static int num_cus = 0;  // idempotent one-time setup; a race only repeats it
+  if (num_cus == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
+      return -4;
+    }
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < 8) {
+      set_error("gemm: cannot query the CU count");
+      return -4;
+    }
+    num_cus = cus - cus % 8;  // a multiple of 8 keeps workgroup id % 8 = XCD for every tile
+  }
+  const int tiles_m = (int)((M + 255) / 256), tiles_n = (N + 255) / 256;
+  const int num_tiles = tiles_m * tiles_n;
+  int group_w = column_group(tiles_n, 256, Kp);
+#ifdef GPTMI_TUNING
+  if (g_group_w > 0) group_w = g_group_w < tiles_n ? g_group_w : tiles_n;
+#endif
+  const int grid = num_tiles < num_cus ? num_tiles : num_cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, st, (const _Float16*)A,
+                     (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n, group_w, ep);
+  return 0;
+}
+
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
@@ -582,8 +921,15 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
   // 128-byte rows per direct load move ~1.5x the bytes per clock of 64-byte rows -- double
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
-  if (M >= 2048 && N >= 256)
+  if (M >= 2048 && N >= 256) {
+    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue, no dropout, no residual: the
+    // streaming kernel (it has neither edge handling nor the generator; with a residual its
+    // epilogue loads queue behind the next tile's operand loads and it measured no faster).
+    if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
+        !(ep.drop.p > 0.f) && (QKV || ep.residual == nullptr))
+      return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  }
   return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 
