@@ -615,7 +615,7 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
 //
 // Load/store counter.  Loads and stores of a wavefront retire in issue order on this ISA.  The
 // loads of the next tile's k-tile 1 are issued BEFORE the epilogue's stores, so waiting for them
-// with vmcnt(16) -- 32 younger stores exist after the epilogue -- does not wait for the stores'
+// with vmcnt(32) -- the epilogue issues exactly 32 stores per lane -- does not wait for the stores'
 // acknowledgements.  The bias is fetched, and waited for, before those loads are issued, so
 // that no compiler-placed wait inside the epilogue falls behind them.  Only whole tiles, no
 // residual, no dropout: the launcher sends everything else to gemm_kernel.
@@ -807,7 +807,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     };
     // publish the k-tile in the other stage and fetch its first fragments (slot 0)
     auto publish_next = [&](bool behind_epilogue, bool fetch) {
-      if (behind_epilogue) wait_vmcnt<16>();
+      // behind an epilogue exactly MB * NB * 4 stores are younger than the loads waited for
+      if (behind_epilogue) wait_vmcnt<MB * NB * 4>();
       else wait_vmcnt<0>();
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (fetch) read_frags(stage ^ 1, 0, 0);
