@@ -279,7 +279,7 @@ def main():
                                        else ", hidden-state output (no LM head)"),
                    "tokens_per_step": tokens, "n_layer": arch["n_layer"], "n_embd": h,
                    "n_head": arch["n_head"]},
-        "roofline": {"kernel": f"gemm_kernel (ffn1: M={tokens} N={4 * h} K={h}, bias+GELU epilogue)",
+        "roofline": {"kernel": f"ffn1 GEMM (gemm_stream_kernel / gemm_kernel: M={tokens} N={4 * h} K={h}, bias+GELU epilogue)",
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16 / 1e12,
                      "unit": "TFLOP/s", "frac": round(achieved * 1e12 / PEAK_FP16, 4),
                      "avg_ms": round(ffn1_ms, 4), "launches": len(ffn1_events),

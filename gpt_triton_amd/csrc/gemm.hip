@@ -923,11 +923,12 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256) {
-    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue, no dropout, no residual: the
-    // streaming kernel (it has neither edge handling nor the generator; with a residual its
-    // epilogue loads queue behind the next tile's operand loads and it measured no faster).
+    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue, no dropout, no residual, no
+    // head-major scatter: the streaming kernel.  It has neither edge handling nor the generator;
+    // with a residual its epilogue loads queue behind the next tile's operand loads and it
+    // measured no faster; the scatter epilogue measured slower inside the model (713 vs 642 us).
     if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
-        !(ep.drop.p > 0.f) && (QKV || ep.residual == nullptr))
+        !(ep.drop.p > 0.f) && !QKV && ep.residual == nullptr)
       return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }
