@@ -8,14 +8,13 @@
 // the q/k/v relayout of matmul_and_split_qkv, kernels.py:347-367, which is done
 // here by the store instead of by three copies.
 //
-// Structure of one workgroup (WM x WN wavefronts):
-//   * a BM x BN output tile; K is walked in steps of BKS (32 or 64) through a
-//     ring of NST LDS stages filled by direct global->LDS loads (16 B per lane,
-//     no VGPR staging).  NST >= 3: the tile after the one being multiplied is
-//     already resident -- the barrier that publishes tile kt+1 sits in front of
-//     the last k-step of tile kt and the first fragments of tile kt+1 are read
-//     right behind it, so no MFMA waits for a barrier plus an LDS round trip.
-//     NST == 2: plain double buffering (all a 256x256x64 stage leaves room for);
+// Structure of one workgroup of gemm_kernel (WM x WN wavefronts):
+//   * a BM x BN output tile; K is walked in steps of BKS (32 or 64) through NST LDS stages
+//     filled by direct global->LDS loads (16 B per lane, no VGPR staging).  The barrier that
+//     publishes k-tile kt+1 sits in front of the LAST k-slice of k-tile kt, whose fragments are
+//     in registers by then; the first fragments of kt+1 are read right behind it and the stage
+//     of kt is refilled with kt+NST while that last slice is multiplied, its load instructions
+//     dealt between the MFMAs.  No MFMA waits for a barrier plus an LDS round trip;
 //   * LDS rows are BKS halves wide; the 16-byte chunks of a row are XOR-swizzled
 //     with a key taken from the row number so that the 16 lanes the LDS serves
 //     per clock (64 banks x 4 B) never share a bank:
@@ -27,10 +26,12 @@
 //   * the epilogue applies bias/GELU in that layout, stages fp32 through LDS
 //     and stores row-major runs (see store_wave_tile);
 //   * workgroup ids are remapped so each XCD (ids are dealt round-robin over
-//     the 8 XCDs) gets a contiguous range of tiles, N fastest: the tiles that
-//     share a row block of A run on the same L2 at the same time.
-#include <type_traits>
-
+//     the 8 XCDs) gets a contiguous range of tiles; inside a group of column tiles whose
+//     weight panels fit the XCD's L2 the column runs fastest, so the tiles that share a row
+//     block of A run on the same L2 at the same time.
+// gemm_stream_kernel (further down) is the persistent form of the 256 x 256 x 64 configuration
+// for whole-tile shapes: one workgroup per CU walks tiles and the pipeline runs across tile
+// boundaries.
 #include "common.h"
 #include "launch.h"
 
