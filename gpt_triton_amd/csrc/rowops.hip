@@ -139,7 +139,10 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
         const float z = (v[i][j] - mean) * rstd;
         to[j] = (T)(z * (float)tw[j] + (float)tb[j]);
       }
-      __builtin_nontemporal_store(to, o + c);
+      // cached (not streaming) store: the [T, H] output is what the following GEMM reads, two
+      // or three times over; it fits the 256 MB memory-side cache, and a GEMM fed from there
+      // instead of HBM ran 12 % faster (its operand loads are only one k-tile ahead)
+      o[c] = to;
     }
   }
 }
