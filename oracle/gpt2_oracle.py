@@ -40,7 +40,9 @@ What pins each function (tests/test_oracle.py):
                against its closed form on the int32 edge values, the keep rate against p, and
                tests/golden/dropout.npz: outputs of the reference's fused_embeddings, fused_ffn
                and flash_attention_v1 with dropout_prob > 0 under Triton's CPU interpreter
-  model        an independently written fp64 torch GPT-2 (HF block order)
+  model        an independently written fp64 torch GPT-2 (HF block order), and the
+               transformers library's GPT2Model (random weights, built locally from a
+               config) through the package's key conversion (test.py:120-133)
 No function of this file is left unpinned.
 """
 import math

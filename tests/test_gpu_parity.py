@@ -401,6 +401,26 @@ def test_gpt2_124m_config0(gpu_device, dtype):
         assert np.abs(host(logits).astype(np.float64) - want_l).max() <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_convert_hf_and_load_model_from_local_directory(gpu_device, dtype, tmp_path):
+    """gpt.py:240-247 with a local directory in place of a hub name: a random HF GPT2Model is
+    saved with save_pretrained, loaded back through convert_hf_and_load_model, and the two
+    forwards are compared the way the reference's test_gpt2 does (test.py:120-133; its
+    tolerance is 1e-1, here 1e-2 in fp32 and 3e-2 with fp16 storage, on |hidden| ~ 5)."""
+    from gpt_triton_amd.gpt import convert_hf_and_load_model
+    from test_oracle import hf_gpt2
+
+    hf = hf_gpt2(vocab_size=97, n_positions=48, n_embd=128, n_layer=2, n_head=2)
+    hf.save_pretrained(str(tmp_path))
+    model, hf_model = convert_hf_and_load_model(str(tmp_path), gpu_device)
+    assert not model.training and model.config.block_size == 48
+    ids = torch.randint(0, 97, (3, 40), device=gpu_device)
+    with torch.no_grad():
+        want = hf_model(ids).last_hidden_state.float().cpu().numpy()
+    got = host(model.to(dtype)(ids)).astype(np.float64)
+    assert np.abs(got - want).max() <= (1e-2 if dtype == torch.float32 else 3e-2)
+
+
 def test_gpt2_layerwise_fp32(K, gpu_device):
     """Every operator of a 3-layer model, each fed the ORACLE's intermediate activations, so
     that no upstream difference is carried along: fp32 storage, tolerance 1e-5 * max|b| (the

@@ -346,6 +346,45 @@ def test_model_composition_vs_independent_fp64_gpt2():
     assert np.abs(bad_h - want_h).max() > 2e-2 * np.abs(want_h).max()
 
 
+def hf_gpt2(seed=1337, **kw):
+    """A randomly initialised HuggingFace GPT2Model (the reference's end-to-end oracle,
+    test.py:120-133), built locally from a config: nothing is downloaded.  Biases and the
+    LayerNorm affine get non-trivial values so that a dropped term shows."""
+    from transformers import GPT2Config, GPT2Model
+
+    torch.manual_seed(seed)
+    cfg = GPT2Config(bos_token_id=None, eos_token_id=None, **kw)
+    hf = GPT2Model(cfg).eval()
+    with torch.no_grad():
+        for name, p in hf.named_parameters():
+            if name.endswith("bias"):
+                p.normal_(0, 0.1)
+            elif "ln_" in name:
+                p.normal_(1, 0.1)
+            else:
+                p.normal_(0, 0.08)
+    return hf
+
+
+def test_model_vs_huggingface_gpt2():
+    """The oracle's forward, fed HF weights through the package's key conversion, against the
+    transformers library's own GPT2Model in fp32 on the CPU.  Tolerance: 1e-2 absolute on
+    hidden states of magnitude ~5 (the oracle rounds every GEMM operand to fp16; the
+    reference's own comparison allows 1e-1, test.py:133)."""
+    from gpt_triton_amd.gpt import convert_huggingface_to_triton
+
+    hf = hf_gpt2(vocab_size=97, n_positions=48, n_embd=128, n_layer=2, n_head=2)
+    ids = torch.randint(0, 97, (3, 40))
+    with torch.no_grad():
+        want = hf(ids).last_hidden_state.numpy()
+    sd, config = convert_huggingface_to_triton(hf.state_dict(), hf.config)
+    assert config.block_size == 48  # n_positions: this transformers has no n_ctx (gpt.py:202)
+    params = {k: v.numpy() for k, v in sd.items()}
+    got = O.gpt2_forward(params, ids.numpy(), config.n_head)
+    assert np.abs(want).max() > 2.0
+    assert np.abs(got - want).max() <= 1e-2
+
+
 # ---------------------------------------------------------------------------
 # dropout: Philox-4x32-10 -> tl.rand -> keep mask (kernels.py:31-34)
 # ---------------------------------------------------------------------------
