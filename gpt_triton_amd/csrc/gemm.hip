@@ -96,6 +96,13 @@ __device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, f4 
                : "memory");
 }
 
+__device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, h8 v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
+               :
+               : "v"(lane_off), "v"(v), "s"(base)
+               : "memory");
+}
+
 // Workgroup barrier that does not drain the vector-memory counter: the
 // compiler's own barrier waits for vmcnt(0), which would serialise the
 // global->LDS prefetch of the younger pipeline stages behind it.
@@ -621,6 +628,45 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
 // that no compiler-placed wait inside the epilogue falls behind them.  Only whole tiles, no
 // residual, no dropout: the launcher sends everything else to gemm_kernel.
 // ---------------------------------------------------------------------------
+// fp16 output, row-major: bias (+GELU) and the rounding to fp16 happen in the accumulator
+// layout, so the transposition through LDS moves 2 bytes per element instead of 4, and a lane
+// gets 8 neighbouring columns back: 16-byte stores, 8 lanes per full 128-byte line.  One pass
+// = 32 rows x 64 columns (both accumulator blocks of a row band) in a 4 KB slab, 16-byte units
+// XOR-swizzled with row & 7.  2 * MB stores per lane in all.
+template <int MB, int NB, bool GELU>
+__device__ __forceinline__ void store_wave_tile16(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+                                                  const EpiDev& ep, int64_t mw0, int nw0, int N,
+                                                  char* slab, int lane) {
+  static_assert(NB == 2, "a pass is two 32-column blocks wide");
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = frow & 7;
+  const int rrow = lane >> 3, runit = lane & 7;  // rrow is also the key of every row it reads
+  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        h4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          if (GELU) z = gelu_new(z);
+          o[e] = (_Float16)z;
+        }
+        *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+      }
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const h8 v =
+          *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
+      store_nt_base(reinterpret_cast<char*>(ep.out) +
+                        ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0) * 2,
+                    lane_byte_off, v);
+    }
+  }
+}
+
 template <int MB, int NB, typename T, bool QKV, bool GELU>
 __device__ __forceinline__ void store_wave_tile32(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
@@ -700,6 +746,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   constexpr int A_IT = 4, B_IT = 4, LPT = A_IT + B_IT;  // 16-byte loads per thread per k-tile
   constexpr int STAGE = (BM + BN) * ROWB;               // 64 KB
   constexpr int SLABS = 2 * STAGE;                      // epilogue slabs start behind the stages
+  constexpr bool HALF_SLABS = sizeof(T) == 2 && !QKV;   // fp16 row-major output: store_wave_tile16
+  constexpr int EPI_STORES = HALF_SLABS ? MB * 2 : MB * NB * 4;  // stores per lane per epilogue
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -808,8 +856,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     };
     // publish the k-tile in the other stage and fetch its first fragments (slot 0)
     auto publish_next = [&](bool behind_epilogue, bool fetch) {
-      // behind an epilogue exactly MB * NB * 4 stores are younger than the loads waited for
-      if (behind_epilogue) wait_vmcnt<MB * NB * 4>();
+      // behind an epilogue exactly EPI_STORES stores are younger than the loads waited for
+      if (behind_epilogue) wait_vmcnt<EPI_STORES>();
       else wait_vmcnt<0>();
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (fetch) read_frags(stage ^ 1, 0, 0);
@@ -870,8 +918,13 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     // ---- epilogue: the next tile's first two k-tiles are landing meanwhile ----
     {
       char* slab = smem + SLABS + wave * 4096;
-      if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
-      else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+      if constexpr (HALF_SLABS) {
+        if (ep.gelu) store_wave_tile16<MB, NB, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        else store_wave_tile16<MB, NB, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+      } else {
+        if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+      }
     }
     if (!has_next) break;
     read_frags(stage, 0, 0);
