@@ -51,6 +51,7 @@ struct EpiDev {
   int d;
   int gelu;
   int vec_ok;  // pointers and N allow 4-element vector accesses
+  int vec8_ok; // fp16 output: N, head size and the output pointers also allow 16-byte stores
   DropoutArgs drop;  // p > 0: dropout between GELU and residual (predicated epilogue only)
 #ifdef GPTMI_TUNING
   unsigned long long* trace;  // tuning builds only: per-workgroup phase time stamps
@@ -80,24 +81,29 @@ __device__ __forceinline__ void lds_dma16_base(const void* base, unsigned lane_o
                : "memory", "m0");
 }
 
-// Streaming store of 4 output elements at (wavefront-uniform 64-bit base) + (32-bit lane
+// Streaming store of 4 or 8 output elements at (wavefront-uniform 64-bit base) + (32-bit lane
 // offset).  Written as assembly because the compiler otherwise materialises one 64-bit address
-// pair per store of an unrolled epilogue and spills.
+// pair per store of an unrolled epilogue and spills.  Two hazards the compiler handles for its
+// own instructions and cannot see inside assembly:
+//   * a scalar register written by a VALU instruction (v_readfirstlane) must not be read by a
+//     memory instruction within the next 5 wait states -- the leading s_nop 4 covers a base
+//     that the compiler had to move out of a vector register;
+//   * a store of more than 64 bits reads its data registers a little after issue -- the
+//     trailing s_nop 1 keeps the next VALU instruction from overwriting them.
 __device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, h4 v) {
-  asm volatile("global_store_dwordx2 %0, %1, %2 nt" : : "v"(lane_off), "v"(v), "s"(base) : "memory");
-}
-__device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, f4 v) {
-  // a store of more than 64 bits reads its data registers a little after issue: the wait states
-  // keep the next VALU instruction from overwriting them (the compiler adds these for its own
-  // stores, it cannot for assembly)
-  asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
+  asm volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2 nt"
                :
                : "v"(lane_off), "v"(v), "s"(base)
                : "memory");
 }
-
+__device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, f4 v) {
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
+               :
+               : "v"(lane_off), "v"(v), "s"(base)
+               : "memory");
+}
 __device__ __forceinline__ void store_nt_base(void* base, unsigned lane_off, h8 v) {
-  asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1"
                :
                : "v"(lane_off), "v"(v), "s"(base)
                : "memory");
@@ -301,6 +307,104 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
   }
 }
 
+// fp16 output without residual, whole tile, vector accesses allowed (and head size % 8 == 0 for
+// the head-major scatter): bias (+GELU) and the rounding to fp16 happen in the accumulator
+// layout, the transposition through the wavefront's slab moves halves (32 rows x 64 columns x
+// 2 bytes per pass, 16-byte units XOR-swizzled with row & 7), and a lane gets 8 neighbouring
+// columns back: 16-byte stores, 8 lanes per 128-byte line -- half the LDS traffic and half the
+// store instructions of the fp32 staging above.  With a residual the sum must stay in fp32 until
+// the one rounding, so those epilogues keep the fp32 slabs.
+template <int MB, int NB, bool QKV, bool GELU>
+__device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const EpiDev& ep,
+                                                  int64_t mw0, int nw0, int N, char* slab,
+                                                  int lane) {
+  static_assert(NB % 2 == 0, "wave tile must be a multiple of 64 columns");
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = frow & 7;
+  const int rrow = lane >> 3, runit = lane & 7;  // rrow is also the key of every row it reads
+  f4 bias_r[NB][4];
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      f4 b = {0.f, 0.f, 0.f, 0.f};
+      if (ep.bias) {
+        const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
+                                                   (nw0 + i * 32 + g * 8 + fhalf * 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
+      }
+      bias_r[i][g] = b;
+    }
+  _Float16* qkv_col[NB / 2];
+  unsigned b0 = 0, l0 = 0;
+  const unsigned Lu = (unsigned)ep.L;
+  const bool step_rows = Lu >= 32u * MB;
+  if (QKV) {
+#pragma unroll
+    for (int i2 = 0; i2 < NB / 2; ++i2)
+      qkv_col[i2] = qkv_column_base<_Float16>(ep, nw0 + i2 * 64 + runit * 8);
+    const unsigned m_first = (unsigned)mw0 + (unsigned)rrow;
+    b0 = m_first / Lu;
+    l0 = m_first - b0 * Lu;
+  }
+  const int64_t batch_stride = (int64_t)ep.heads * ep.L * ep.d;
+  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+#pragma unroll
+    for (int i2 = 0; i2 < NB / 2; ++i2) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int i = i2 * 2 + ii;
+          h4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+            if (GELU) z = gelu_new(z);
+            o[e] = (_Float16)z;
+          }
+          *reinterpret_cast<h4*>(slab + frow * 128 + (((ii * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+        }
+      // all four reads first: the stores are assembly with a memory clobber, which no LDS
+      // read may cross, so reading inside the store loop would expose one LDS latency per store
+      h8 vv[4];
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        vv[rr] =
+            *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const h8 v = vv[rr];
+        if constexpr (QKV) {
+          unsigned b, l;
+          if (step_rows) {
+            b = b0;
+            l = l0 + (unsigned)(j * 32 + rr * 8);
+            if (l >= Lu) { l -= Lu; ++b; }
+          } else {
+            const unsigned m = (unsigned)mw0 + (unsigned)(j * 32 + rr * 8 + rrow);
+            b = m / Lu;
+            l = m - b * Lu;
+          }
+          _Float16* dst = qkv_col[i2] + ((int64_t)b * batch_stride + (int64_t)l * ep.d);
+          __builtin_nontemporal_store(v, reinterpret_cast<h8*>(dst));
+        } else {
+          // wavefront-uniform 64-bit part in scalar registers + one 32-bit lane offset.  mw0 and
+          // nw0 derive from a wavefront index the kernel made provably uniform, so this is
+          // scalar arithmetic: a base produced by v_readfirstlane right in front of the store
+          // would need five wait states the compiler does not insert for assembly, and the
+          // store would now and then go out with the previous base.
+          store_nt_base(reinterpret_cast<char*>(ep.out) +
+                            ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0 + i2 * 64) * 2,
+                        lane_byte_off, v);
+        }
+      }
+    }
+  }
+}
+
 template <int MB, int NB, typename T, bool QKV>
 __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDev& ep,
                                                 int64_t mw0, int nw0, int M, int N, bool fast,
@@ -313,6 +417,13 @@ __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDe
       if (ep.gelu) { if (res) GPTMI_EPI_DROP(true, true); else GPTMI_EPI_DROP(true, false); }
       else { if (res) GPTMI_EPI_DROP(false, true); else GPTMI_EPI_DROP(false, false); }
 #undef GPTMI_EPI_DROP
+      return;
+    }
+  }
+  if constexpr (sizeof(T) == 2) {
+    if (fast && !res && ep.vec8_ok) {
+      if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, ep, mw0, nw0, N, slab, lane);
+      else store_wave_tile_h<MB, NB, QKV, false>(acc, ep, mw0, nw0, N, slab, lane);
       return;
     }
   }
@@ -364,7 +475,10 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // provably wavefront-uniform, so that everything derived from the wavefront's sub-tile origin
+  // (the base addresses of the epilogue's stores) is scalar arithmetic in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % WM, wn = wave / WM;
 #ifdef GPTMI_TUNING
   const unsigned long long t_start = __builtin_amdgcn_s_memtime();
@@ -656,14 +770,17 @@ __device__ __forceinline__ void store_wave_tile16(f16v (&acc)[NB][MB], const f4 
         }
         *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
       }
+    // all four reads first: the stores are assembly with a memory clobber, which no LDS read
+    // may cross, so reading inside the store loop would expose one LDS latency per store
+    h8 vv[4];
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      const h8 v =
-          *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
+    for (int rr = 0; rr < 4; ++rr)
+      vv[rr] = *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
       store_nt_base(reinterpret_cast<char*>(ep.out) +
                         ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0) * 2,
-                    lane_byte_off, v);
-    }
+                    lane_byte_off, vv[rr]);
   }
 }
 
@@ -982,7 +1099,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     // with a residual its epilogue loads queue behind the next tile's operand loads and it
     // measured no faster; the scatter epilogue measured slower inside the model (713 vs 642 us).
     if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
-        !(ep.drop.p > 0.f) && !QKV && ep.residual == nullptr)
+        (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && !QKV && ep.residual == nullptr)
       return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }
@@ -1020,6 +1137,9 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const G
   const bool vec = (N % 4) == 0 && aligned(e.bias) && aligned(e.residual) && aligned(e.out) &&
                    aligned(e.q) && aligned(e.k) && aligned(e.v);
   ep.vec_ok = vec ? 1 : 0;
+  auto aligned16 = [&](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  ep.vec8_ok = vec && e.f16 && (N % 8) == 0 && aligned16(e.out) && aligned16(e.q) &&
+               aligned16(e.k) && aligned16(e.v) && (!e.qkv || (e.d % 8) == 0);
   if (e.f16)
     return e.qkv ? launch_shape<_Float16, true>(A, Bt, M, N, Kp, ep, st)
                  : launch_shape<_Float16, false>(A, Bt, M, N, Kp, ep, st);

@@ -249,6 +249,25 @@ def test_matmul_and_split_qkv(K, gpu_device, dtype, B, L, heads, d):
         check(host(got), want, dtype, "qkv")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("B,L,heads,d", [(9, 300, 12, 64), (9, 300, 12, 72), (9, 300, 12, 20)])
+def test_matmul_and_split_qkv_big_tiles(K, gpu_device, dtype, B, L, heads, d):
+    """M = 2700 rows: the 256 x 256 kernel with whole tiles, a ragged last row of tiles and
+    batch boundaries inside a tile; head sizes that allow 16-byte scatter stores (64, 72)
+    and one that does not (20)."""
+    r = np.random.default_rng(17)
+    h = heads * d
+    x = r.standard_normal((B, L, h)).astype(NP[dtype])
+    w = (0.03 * r.standard_normal((h, 3 * h))).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(3 * h)).astype(NP[dtype])
+    q, k, v = K.matmul_and_split_qkv(dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device),
+                                     heads)
+    wq, wk, wv = O.matmul_and_split_qkv(x, w, b, heads)
+    for got, want in ((q, wq), (k, wk), (v, wv)):
+        assert got.shape == (B, heads, L, d) and got.is_contiguous()
+        check(host(got), want, dtype, "qkv")
+
+
 # ----------------------------------------------------------------------------- attention
 def attn_inputs(B, N, L, D, dtype, gaussian, seed=1337):
     r = np.random.default_rng(seed)
