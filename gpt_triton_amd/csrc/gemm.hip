@@ -314,27 +314,15 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
 // columns back: 16-byte stores, 8 lanes per 128-byte line -- half the LDS traffic and half the
 // store instructions of the fp32 staging above.  With a residual the sum must stay in fp32 until
 // the one rounding, so those epilogues keep the fp32 slabs.
+// bias_r[i][g] = bias of the lane's 4 columns nw0 + 32 i + 8 g + 4 (lane / 32) + 0..3.
+// (NB / 2) * MB * 4 stores per lane.
 template <int MB, int NB, bool QKV, bool GELU>
-__device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const EpiDev& ep,
-                                                  int64_t mw0, int nw0, int N, char* slab,
-                                                  int lane) {
+__device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+                                                  const EpiDev& ep, int64_t mw0, int nw0, int N,
+                                                  char* slab, int lane) {
   static_assert(NB % 2 == 0, "wave tile must be a multiple of 64 columns");
   const int frow = lane & 31, fhalf = lane >> 5, fkey = frow & 7;
   const int rrow = lane >> 3, runit = lane & 7;  // rrow is also the key of every row it reads
-  f4 bias_r[NB][4];
-#pragma unroll
-  for (int i = 0; i < NB; ++i)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      f4 b = {0.f, 0.f, 0.f, 0.f};
-      if (ep.bias) {
-        const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
-                                                   (nw0 + i * 32 + g * 8 + fhalf * 4));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-      }
-      bias_r[i][g] = b;
-    }
   _Float16* qkv_col[NB / 2];
   unsigned b0 = 0, l0 = 0;
   const unsigned Lu = (unsigned)ep.L;
@@ -422,8 +410,23 @@ __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDe
   }
   if constexpr (sizeof(T) == 2) {
     if (fast && !res && ep.vec8_ok) {
-      if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, ep, mw0, nw0, N, slab, lane);
-      else store_wave_tile_h<MB, NB, QKV, false>(acc, ep, mw0, nw0, N, slab, lane);
+      const int fhalf = lane >> 5;
+      f4 bias_r[NB][4];
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f4 b = {0.f, 0.f, 0.f, 0.f};
+          if (ep.bias) {
+            const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
+                                                       (nw0 + i * 32 + g * 8 + fhalf * 4));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
+          }
+          bias_r[i][g] = b;
+        }
+      if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+      else store_wave_tile_h<MB, NB, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       return;
     }
   }
@@ -732,58 +735,17 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
 // two workgroups while the stores of the one that ended drain (measured: 231 of 256 CUs busy
 // on average with one workgroup per tile, 251 when the kernel stores nothing).
 //
-// LDS: stages at [0, 128 KB), epilogue slabs behind them (8 wavefronts x 4 KB: one 32 x 32 fp32
-// block, 16-byte units XOR-swizzled with (row >> 1) & 7), so the epilogue never touches a stage.
+// LDS: stages at [0, 128 KB), epilogue slabs behind them (8 wavefronts x 4 KB: 32 rows x 64
+// halves for fp16 output, store_wave_tile_h; one 32 x 32 fp32 block for fp32 output, 16-byte
+// units XOR-swizzled with (row >> 1) & 7), so the epilogue never touches a stage.
 //
 // Load/store counter.  Loads and stores of a wavefront retire in issue order on this ISA.  The
 // loads of the next tile's k-tile 1 are issued BEFORE the epilogue's stores, so waiting for them
-// with vmcnt(32) -- the epilogue issues exactly 32 stores per lane -- does not wait for the stores'
-// acknowledgements.  The bias is fetched, and waited for, before those loads are issued, so
+// with vmcnt(EPI_STORES) -- the epilogue issues exactly 16 (fp16) or 32 (fp32) stores per lane --
+// does not wait for the stores' acknowledgements.  The bias is fetched, and waited for, before those loads are issued, so
 // that no compiler-placed wait inside the epilogue falls behind them.  Only whole tiles, no
 // residual, no dropout: the launcher sends everything else to gemm_kernel.
 // ---------------------------------------------------------------------------
-// fp16 output, row-major: bias (+GELU) and the rounding to fp16 happen in the accumulator
-// layout, so the transposition through LDS moves 2 bytes per element instead of 4, and a lane
-// gets 8 neighbouring columns back: 16-byte stores, 8 lanes per full 128-byte line.  One pass
-// = 32 rows x 64 columns (both accumulator blocks of a row band) in a 4 KB slab, 16-byte units
-// XOR-swizzled with row & 7.  2 * MB stores per lane in all.
-template <int MB, int NB, bool GELU>
-__device__ __forceinline__ void store_wave_tile16(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
-                                                  const EpiDev& ep, int64_t mw0, int nw0, int N,
-                                                  char* slab, int lane) {
-  static_assert(NB == 2, "a pass is two 32-column blocks wide");
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = frow & 7;
-  const int rrow = lane >> 3, runit = lane & 7;  // rrow is also the key of every row it reads
-  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
-#pragma unroll
-  for (int j = 0; j < MB; ++j) {
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        h4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
-          if (GELU) z = gelu_new(z);
-          o[e] = (_Float16)z;
-        }
-        *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
-      }
-    // all four reads first: the stores are assembly with a memory clobber, which no LDS read
-    // may cross, so reading inside the store loop would expose one LDS latency per store
-    h8 vv[4];
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr)
-      vv[rr] = *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr)
-      store_nt_base(reinterpret_cast<char*>(ep.out) +
-                        ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0) * 2,
-                    lane_byte_off, vv[rr]);
-  }
-}
-
 template <int MB, int NB, typename T, bool QKV, bool GELU>
 __device__ __forceinline__ void store_wave_tile32(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
@@ -863,8 +825,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   constexpr int A_IT = 4, B_IT = 4, LPT = A_IT + B_IT;  // 16-byte loads per thread per k-tile
   constexpr int STAGE = (BM + BN) * ROWB;               // 64 KB
   constexpr int SLABS = 2 * STAGE;                      // epilogue slabs start behind the stages
-  constexpr bool HALF_SLABS = sizeof(T) == 2 && !QKV;   // fp16 row-major output: store_wave_tile16
-  constexpr int EPI_STORES = HALF_SLABS ? MB * 2 : MB * NB * 4;  // stores per lane per epilogue
+  constexpr bool HALF_SLABS = sizeof(T) == 2;           // fp16 output: store_wave_tile_h
+  constexpr int EPI_STORES = HALF_SLABS ? MB * NB * 2 : MB * NB * 4;  // stores per lane per epilogue
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1036,8 +998,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     {
       char* slab = smem + SLABS + wave * 4096;
       if constexpr (HALF_SLABS) {
-        if (ep.gelu) store_wave_tile16<MB, NB, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
-        else store_wave_tile16<MB, NB, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        else store_wave_tile_h<MB, NB, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       } else {
         if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
         else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
@@ -1094,12 +1056,12 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256) {
-    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue, no dropout, no residual, no
-    // head-major scatter: the streaming kernel.  It has neither edge handling nor the generator;
-    // with a residual its epilogue loads queue behind the next tile's operand loads and it
-    // measured no faster; the scatter epilogue measured slower inside the model (713 vs 642 us).
+    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue (16-byte stores for fp16), no
+    // dropout, no residual: the streaming kernel.  It has neither edge handling nor the
+    // generator; with a residual its epilogue loads queue behind the next tile's operand loads
+    // and it measured no faster.
     if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
-        (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && !QKV && ep.residual == nullptr)
+        (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr)
       return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }

@@ -250,11 +250,14 @@ def test_matmul_and_split_qkv(K, gpu_device, dtype, B, L, heads, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-@pytest.mark.parametrize("B,L,heads,d", [(9, 300, 12, 64), (9, 300, 12, 72), (9, 300, 12, 20)])
+@pytest.mark.parametrize("B,L,heads,d", [(9, 300, 12, 64), (9, 300, 12, 72), (9, 300, 12, 20),
+                                         (8, 320, 12, 64), (64, 40, 12, 64), (8, 320, 8, 32)])
 def test_matmul_and_split_qkv_big_tiles(K, gpu_device, dtype, B, L, heads, d):
     """M = 2700 rows: the 256 x 256 kernel with whole tiles, a ragged last row of tiles and
     batch boundaries inside a tile; head sizes that allow 16-byte scatter stores (64, 72)
-    and one that does not (20)."""
+    and one that does not (20).  M = 2560 rows with 3 * heads * d a multiple of 256: the
+    streaming kernel, with sequences longer (320) and shorter (40) than a wavefront's 128
+    rows, i.e. both ways of finding (batch, position) of a row."""
     r = np.random.default_rng(17)
     h = heads * d
     x = r.standard_normal((B, L, h)).astype(NP[dtype])
