@@ -43,10 +43,10 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
 }
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
-# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (947.1 MB after scaling by
-# the copy kernel of --traffic-calibration) + WRITE_SIZE (1126.2 MB); the counters cannot be read
+# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (952.9 MB after scaling by
+# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.8 MB); the counters cannot be read
 # from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
-FFN1_TRAFFIC_BYTES = 2.073e9
+FFN1_TRAFFIC_BYTES = 1.897e9
 
 
 def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
