@@ -321,8 +321,11 @@ __device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 
                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
                                                   char* slab, int lane) {
   static_assert(NB % 2 == 0, "wave tile must be a multiple of 64 columns");
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = frow & 7;
-  const int rrow = lane >> 3, runit = lane & 7;  // rrow is also the key of every row it reads
+  // key (row >> 1) & 7: the 32 rows x 2 lanes of one 8-byte write then cover 16 distinct
+  // 16-byte slots of the 256-byte bank window twice -- the minimum for 512 bytes
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int rrow = lane >> 3, runit = lane & 7;
+  const int rkey = rrow >> 1;  // key of row 8 rr + rrow = rkey ^ 4 (rr & 1)
   _Float16* qkv_col[NB / 2];
   unsigned b0 = 0, l0 = 0;
   const unsigned Lu = (unsigned)ep.L;
@@ -360,8 +363,8 @@ __device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 
       h8 vv[4];
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr)
-        vv[rr] =
-            *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 + ((runit ^ rrow) << 4));
+        vv[rr] = *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 +
+                                              ((runit ^ rkey ^ ((rr & 1) * 4)) << 4));
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const h8 v = vv[rr];
@@ -390,6 +393,59 @@ __device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 
         }
       }
     }
+  }
+}
+
+// fp16 output WITH residual, whole tile, 16-byte accesses allowed: the wavefront's 128 x 64
+// residual sub-tile was brought into LDS by direct loads (rows 0..63 at res_lo while the last
+// k-tile was multiplied, rows 64..127 at res_hi right after the loop; 128 bytes per row, 16-byte
+// units XOR-swizzled with (row >> 1) & 7), so the epilogue reads it in the accumulator layout, adds it
+// in fp32 behind bias (+GELU) -- the reference's order -- rounds once, and finishes like
+// store_wave_tile_h.  No global load is waited for between the stores: the two waits below count
+// exactly what is younger than the residual loads (the second half's 8 loads; then the 8
+// stores of row bands 0 and 1).
+template <int MB, int NB, bool GELU>
+__device__ __forceinline__ void store_wave_tile_rl(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
+                                                   const char* res_lo, const char* res_hi,
+                                                   char* slab, int lane) {
+  static_assert(MB == 4 && NB == 2, "128 x 64 sub-tile");
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int rrow = lane >> 3, runit = lane & 7, rkey = rrow >> 1;
+  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+    if (j == 0 || j == 2) wait_vmcnt<8>();
+    const char* rb = (j < 2 ? res_lo : res_hi) + ((j & 1) * 32 + frow) * 128 + fhalf * 8;
+    h4 r[NB][4];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        r[i][g] = *reinterpret_cast<const h4*>(rb + (((i * 4 + g) ^ fkey) << 4));
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        h4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          if (GELU) z = gelu_new(z);
+          o[e] = (_Float16)(z + (float)r[i][g][e]);
+        }
+        *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+      }
+    h8 vv[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+      vv[rr] = *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 +
+                                            ((runit ^ rkey ^ ((rr & 1) * 4)) << 4));
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+      store_nt_base(reinterpret_cast<char*>(ep.out) +
+                        ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0) * 2,
+                    lane_byte_off, vv[rr]);
   }
 }
 
@@ -454,7 +510,8 @@ __device__ __forceinline__ int xcd_tile(int pid, int num_tiles) {
 
 // WPE = wavefronts per SIMD the register allocation must leave room for (two
 // 4-wavefront workgroups per CU need 2).
-template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
+template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV,
+          bool RESLDS = false>
 __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
     int tiles_m, int tiles_n, int group_w, EpiDev ep) {
@@ -475,6 +532,12 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   static_assert(TM % 32 == 0 && TN % 64 == 0, "wave tile must be 32 x 64 aligned");
   static_assert(NST * STAGE >= WM * WN * EP_SLAB, "epilogue staging does not fit");
   static_assert((NST - 2) * LPT <= 63, "vmcnt range");
+  // RESLDS (launched with a residual; 32 KB of LDS behind the stages for the epilogue slabs):
+  // workgroups whose tile is whole bring the residual tile into the operand stages as these fall
+  // free and run store_wave_tile_rl; tiles on the matrix edge take the predicated epilogue.
+  static_assert(!RESLDS || (sizeof(T) == 2 && !QKV && NST == 2 && BM == 256 && BN == 256 &&
+                            WM == 2 && WN == 4 && BKS == 64),
+                "residual through LDS: the 256 x 256 x 64 configuration, fp16 row-major output");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -595,6 +658,26 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #else
   constexpr bool loads = true;
 #endif
+  // Residual through LDS.  Half h = rows 64 h .. 64 h + 63 of the wavefront's sub-tile goes
+  // to this wavefront's own 8 KB of operand stage `stg`: 8 direct loads of 8 rows, lane l of
+  // load q fetching 16-byte unit (l % 8) ^ key of row r = 8 q + l / 8, key = (r >> 1) & 7 =
+  // (l / 16) ^ 4 (q & 1), so that unit u of row r lies at position u ^ key of the row's 128 bytes.
+  const bool res_lds =
+      RESLDS && ep.residual != nullptr && ep.vec_ok && n0 + BN <= N && m0 + BM <= M;
+  unsigned res_lane_off[2];
+#pragma unroll
+  for (int odd = 0; odd < 2; ++odd)
+    res_lane_off[odd] = ((unsigned)(lane >> 3) * (unsigned)N +
+                         (unsigned)(((lane & 7) ^ (lane >> 4) ^ (odd * 4)) * 8)) * 2u;
+  auto issue_res_half = [&](int h, int stg) {
+    const char* base = (const char*)ep.residual +
+                       (((int64_t)m0 + wm * TM + h * 64) * N + (n0 + wn * TN)) * 2;
+    const unsigned lds = (unsigned)(uintptr_t)smem + (unsigned)stg * STAGE + (unsigned)wave * 8192u;
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      lds_dma16_base(base + (int64_t)q * 8 * N * 2, res_lane_off[q & 1], lds + q * 1024);
+  };
+
   // Pipeline.  NST k-tiles are in LDS or on their way at any time.  Fragments of the next
   // k-slice are requested before the MFMAs of the current one issue (the scheduling fences keep
   // the compiler from sinking the reads behind the MFMAs again).  In front of the LAST k-slice of
@@ -645,6 +728,13 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #endif
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (RESLDS) {
+      // the stage of k-tile KT-2 fell free at the barrier in front of its last slice
+      if (res_lds && kt == KT - 2) {
+        issue_res_half(0, kt % NST);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
 
   // ---- epilogue -----------------------------------------------------------
@@ -665,8 +755,47 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #else
   block_barrier();  // every wavefront is done reading the operand stages
   const bool fast = ep.vec_ok && n0 + BN <= N && m0 + BM <= M;
-  store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM, n0 + wn * TN, M, N, fast,
-                                  smem + wave * EP_SLAB, lane);
+  bool stored = false;
+  if constexpr (RESLDS) {
+    if (res_lds) {
+      const int nw0 = n0 + wn * TN, fhalf = lane >> 5;
+      // the bias first, and waited for, so that no compiler-placed wait inside the epilogue
+      // falls behind the second half's loads
+      f4 bias_r[NB][4];
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f4 b = {0.f, 0.f, 0.f, 0.f};
+          if (ep.bias) {
+            const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
+                                                       (nw0 + i * 32 + g * 8 + fhalf * 4));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
+          }
+          bias_r[i][g] = b;
+        }
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
+      const int s_lo = (KT - 2) % NST, s_hi = (KT - 1) % NST;
+      issue_res_half(1, s_hi);
+      const char* res_lo = smem + s_lo * STAGE + wave * 8192;
+      const char* res_hi = smem + s_hi * STAGE + wave * 8192;
+      char* slab = smem + NST * STAGE + wave * 4096;
+      if (ep.gelu)
+        store_wave_tile_rl<MB, NB, true>(acc, bias_r, ep, (int64_t)m0 + wm * TM, nw0, N, res_lo,
+                                         res_hi, slab, lane);
+      else
+        store_wave_tile_rl<MB, NB, false>(acc, bias_r, ep, (int64_t)m0 + wm * TM, nw0, N, res_lo,
+                                          res_hi, slab, lane);
+      stored = true;
+    }
+  }
+  if (!stored)
+    store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM, n0 + wn * TN, M, N, fast,
+                                    smem + wave * EP_SLAB, lane);
 #endif
 #ifdef GPTMI_TUNING
   if (ep.trace && tid == 0) {
@@ -700,11 +829,12 @@ inline int column_group(int tiles_n, int bn, int Kp) {
   return (tiles_n + groups - 1) / groups;
 }
 
-template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV>
+template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV,
+          bool RESLDS = false>
 int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                hipStream_t st) {
-  auto kern = gemm_kernel<BM, BN, WM, WN, BKS, NST, WPE, T, QKV>;
-  constexpr int smem = NST * (BM + BN) * BKS * 2;
+  auto kern = gemm_kernel<BM, BN, WM, WN, BKS, NST, WPE, T, QKV, RESLDS>;
+  constexpr int smem = NST * (BM + BN) * BKS * 2 + (RESLDS ? WM * WN * 4096 : 0);
   static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1063,6 +1193,12 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
         (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr)
       return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
+    // fp16 with a residual, no dropout: whole tiles fetch the residual through LDS
+    if constexpr (sizeof(T) == 2 && !QKV) {
+      if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&
+          (((uintptr_t)ep.residual) & 15) == 0)
+        return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV, true>(A, Bt, M, N, Kp, ep, st);
+    }
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }
   return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
