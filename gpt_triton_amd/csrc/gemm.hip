@@ -52,6 +52,7 @@ struct EpiDev {
   int gelu;
   int vec_ok;  // pointers and N allow 4-element vector accesses
   int vec8_ok; // fp16 output: N, head size and the output pointers also allow 16-byte stores
+  int m_off;   // head-major scatter: row 0 of this launch is row m_off of the [B*L] token rows
   DropoutArgs drop;  // p > 0: dropout between GELU and residual (predicated epilogue only)
 #ifdef GPTMI_TUNING
   unsigned long long* trace;  // tuning builds only: per-workgroup phase time stamps
@@ -793,9 +794,12 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       stored = true;
     }
   }
-  if (!stored)
-    store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM, n0 + wn * TN, M, N, fast,
-                                    smem + wave * EP_SLAB, lane);
+  if (!stored) {
+    // the scatter finds (batch, position) from the token row: launch-relative row + m_off
+    const int moff = QKV ? ep.m_off : 0;
+    store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM + moff, n0 + wn * TN, M + moff,
+                                    N, fast, smem + wave * EP_SLAB, lane);
+  }
 #endif
 #ifdef GPTMI_TUNING
   if (ep.trace && tid == 0) {
@@ -1144,19 +1148,11 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   }
 }
 
-template <int WM, int WN, typename T, bool QKV>
-int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
-                  hipStream_t st) {
-  auto kern = gemm_stream_kernel<WM, WN, T, QKV>;
-  constexpr int smem = 2 * 512 * 128 + 8 * 4096;  // 160 KB: two stages + the epilogue slabs
+// CUs of the current device rounded down to a multiple of 8 (workgroup id % 8 = XCD for every
+// tile of a persistent launch), or a negative error code.
+inline int cu_count() {
   static int num_cus = 0;  // idempotent one-time setup; a race only repeats it
   if (num_cus == 0) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
-      return -4;
-    }
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
@@ -1164,8 +1160,28 @@ int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const
       set_error("gemm: cannot query the CU count");
       return -4;
     }
-    num_cus = cus - cus % 8;  // a multiple of 8 keeps workgroup id % 8 = XCD for every tile
+    num_cus = cus - cus % 8;
   }
+  return num_cus;
+}
+
+template <int WM, int WN, typename T, bool QKV>
+int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+                  hipStream_t st) {
+  auto kern = gemm_stream_kernel<WM, WN, T, QKV>;
+  constexpr int smem = 2 * 512 * 128 + 8 * 4096;  // 160 KB: two stages + the epilogue slabs
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  const int num_cus = cu_count();
+  if (num_cus < 0) return num_cus;
   const int tiles_m = (int)((M + 255) / 256), tiles_n = (N + 255) / 256;
   const int num_tiles = tiles_m * tiles_n;
   int group_w = column_group(tiles_n, 256, Kp);
@@ -1191,8 +1207,26 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     // generator; with a residual its epilogue loads queue behind the next tile's operand loads
     // and it measured no faster.
     if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
-        (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr)
-      return launch_stream<2, 4, T, QKV>(A, Bt, M, N, Kp, ep, st);
+        (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr) {
+      // Every persistent workgroup walks ceil(tiles / CUs) tiles, so a few tiles beyond a whole
+      // number of rounds cost a full round.  Then the last rows leave the persistent launch --
+      // as many row tiles stay as fill whole rounds -- and go to the small-tile kernel, whose
+      // many short workgroups spread over all CUs (headline ffn1: 7200 tiles = 28 rounds + 32
+      // tiles; 597 of the 600 row tiles stay, 768 rows follow as 144 tiles of 128 x 128).
+      const int cus = cu_count();
+      if (cus < 0) return cus;
+      const int64_t tiles_m = M / 256, tiles_n = N / 256, tiles = tiles_m * tiles_n;
+      const int64_t rounds = tiles / cus, rem = tiles % cus;
+      int64_t m_head = M;
+      if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;
+      int rc = launch_stream<2, 4, T, QKV>(A, Bt, m_head, N, Kp, ep, st);
+      if (rc != 0 || m_head == M) return rc;
+      EpiDev tail = ep;
+      if (QKV) tail.m_off = ep.m_off + (int)m_head;
+      else tail.out = (T*)ep.out + m_head * N;
+      return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>((const _Float16*)A + m_head * Kp, Bt,
+                                                          M - m_head, N, Kp, tail, st);
+    }
     // fp16 with a residual, no dropout: whole tiles fetch the residual through LDS
     if constexpr (sizeof(T) == 2 && !QKV) {
       if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&

@@ -514,6 +514,29 @@ def test_full_size_ffn_rows(K, gpu_device):
     assert (y.float().abs().sum(dim=1) > 0).all()
 
 
+def test_full_size_qkv_split(K, gpu_device):
+    """The headline qkv product: [512, 300, 768] fp16 @ [768, 2304] + b, scattered to q, k, v
+    [512, 12, 300, 64].  600 x 9 tiles are 21 rounds of 256 workgroups and 24 tiles more, so
+    the launcher sends the last 768 token rows to the small-tile kernel with a row offset:
+    sampled sequences from the head, from both sides of that seam (row 152832 = sequence 509,
+    position 132) and the last one are compared with the oracle."""
+    g = torch.Generator(device="cpu").manual_seed(3)
+    B, L, heads, d = 512, 300, 12, 64
+    h = heads * d
+    x = torch.randn((B, L, h), generator=g).half()
+    w = (0.03 * torch.randn((h, 3 * h), generator=g)).half()
+    b = (0.1 * torch.randn(3 * h, generator=g)).half()
+    q, k, v = K.matmul_and_split_qkv(x.to(gpu_device), w.to(gpu_device), b.to(gpu_device), heads)
+    assert q.shape == (B, heads, L, d) and q.is_contiguous()
+    for t in (q, k, v):
+        assert torch.isfinite(t).all()
+    seqs = [0, 1, 255, 508, 509, 510, 511]
+    wq, wk, wv = O.matmul_and_split_qkv(x[seqs].numpy(), w.numpy(), b.numpy(), heads)
+    idx = torch.tensor(seqs, device=gpu_device)
+    for got, want, name in ((q, wq, "q"), (k, wk, "k"), (v, wv, "v")):
+        check(got[idx].cpu().numpy(), want, torch.float16, f"qkv full size {name}")
+
+
 def test_full_size_attention_heads(K, gpu_device):
     """BASELINE config 2: q, k, v [512, 12, 300, 64] fp16; (batch, head) pairs are independent."""
     g = torch.Generator(device="cpu").manual_seed(2)
