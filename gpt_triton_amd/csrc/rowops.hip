@@ -147,6 +147,61 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
   }
 }
 
+// The same for rows of exactly 32 * CH chunks (H = 768: 96 chunks of 8 halves): half a wavefront
+// per row, two rows per wavefront.  Every lane then has work in every chunk (with 64 lanes a
+// quarter of them idle in the second chunk of a 96-chunk row) and a wavefront keeps twice the rows
+// in flight.  Sums run over 32 lanes (shuffle distances 16..1 never leave a half).
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void layernorm_half_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
+    T* __restrict__ out, int64_t M, int H, float eps) {
+  typedef typename Vec<T>::type V;
+  constexpr int VN = Vec<T>::N;
+  const int sub = threadIdx.x & 31;
+  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  if (row >= M) return;
+  const V* xr = reinterpret_cast<const V*>(x + row * H);
+  float v[CH][VN];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    V t = __builtin_nontemporal_load(xr + sub + i * 32);
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      v[i][j] = (float)t[j];
+      s += v[i][j];
+    }
+  }
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+  const float mean = s / (float)H;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i)
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const float d = v[i][j] - mean;
+      q += d * d;
+    }
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, kWave);
+  const float rstd = 1.0f / sqrtf(q / (float)H + eps);
+  const V* wv = reinterpret_cast<const V*>(w);
+  const V* bv = reinterpret_cast<const V*>(b);
+  V* o = reinterpret_cast<V*>(out + row * H);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = sub + i * 32;
+    V tw = wv[c], tb = bv[c], to;
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const float z = (v[i][j] - mean) * rstd;
+      to[j] = (T)(z * (float)tw[j] + (float)tb[j]);
+    }
+    o[c] = to;  // cached store, as above
+  }
+}
+
 // Any H (no alignment requirement): the row is re-read from cache per pass.
 template <typename T>
 __global__ __launch_bounds__(256) void layernorm_scalar_kernel(
@@ -326,6 +381,14 @@ static void ln_go(const void* x, const void* w, const void* b, void* out, int64_
                      (T*)out, M, H, eps);
 }
 
+template <typename T, int CH>
+static void ln_half_go(const void* x, const void* w, const void* b, void* out, int64_t M,
+                       int H, float eps, hipStream_t st) {
+  hipLaunchKernelGGL((layernorm_half_kernel<T, CH>), dim3((unsigned)((M + 7) / 8)),
+                     dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
+                     (T*)out, M, H, eps);
+}
+
 template <typename T>
 static int launch_layernorm_t(const void* x, const void* w, const void* b, void* out,
                               int64_t M, int H, float eps, hipStream_t st) {
@@ -333,6 +396,16 @@ static int launch_layernorm_t(const void* x, const void* w, const void* b, void*
   const bool aligned = (H % VN) == 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0 &&
                        ((uintptr_t)out % 16) == 0;
+  if (aligned && (H / VN) % 32 == 0) {
+    switch (H / VN / 32) {
+      case 1: ln_half_go<T, 1>(x, w, b, out, M, H, eps, st); return 0;
+      case 2: ln_half_go<T, 2>(x, w, b, out, M, H, eps, st); return 0;
+      case 3: ln_half_go<T, 3>(x, w, b, out, M, H, eps, st); return 0;
+      case 4: ln_half_go<T, 4>(x, w, b, out, M, H, eps, st); return 0;
+      case 6: ln_half_go<T, 6>(x, w, b, out, M, H, eps, st); return 0;
+      default: break;
+    }
+  }
   const int need = aligned ? (H / VN + 63) / 64 : 1 << 30;
   if (need <= 1) ln_go<T, 1>(x, w, b, out, M, H, eps, st);
   else if (need <= 2) ln_go<T, 2>(x, w, b, out, M, H, eps, st);
