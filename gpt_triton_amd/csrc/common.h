@@ -27,6 +27,19 @@ __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
   return v;
 }
+// The same over aligned groups of G lanes (G = 64: the wavefront; G = 32: each half on its own).
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+template <int G>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
 
 // tanh-form GELU of the reference (kernels.py:15-26): 0.5 x (1 + tanh(u)) with
 // tanh(u) = 2 sigmoid(2u) - 1, u = sqrt(2/pi) (x + 0.044715 x^3).  Algebraically

@@ -21,14 +21,14 @@ template <> struct Vec<float> {
 // (reference: fused_embeddings_kernel, kernels.py:37-72).  The add is done in
 // fp32 and rounded once, which equals one add in the storage dtype.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int LPR>
 __global__ __launch_bounds__(256) void embed_vec_kernel(
     const int64_t* __restrict__ ids, const T* __restrict__ wte,
     const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H) {
   typedef typename Vec<T>::type V;
   constexpr int VN = Vec<T>::N;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & (LPR - 1);  // LPR lanes per token, as in the LayerNorm kernel
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
   if (row >= rows) return;
   const int64_t tok = ids[row];
   const int64_t pos = row % L;
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void embed_vec_kernel(
   const V* b = reinterpret_cast<const V*>(wpe + pos * H);
   V* o = reinterpret_cast<V*>(out + row * H);
   const int nchunks = H / VN;
-  for (int c = lane; c < nchunks; c += 64) {
+  for (int c = lane; c < nchunks; c += LPR) {
     V va = a[c], vb = b[c], vo;
 #pragma unroll
     for (int j = 0; j < VN; ++j) vo[j] = (T)((float)va[j] + (float)vb[j]);
@@ -83,15 +83,20 @@ __global__ __launch_bounds__(256) void embed_dropout_kernel(
 // LayerNorm (reference: fused_layer_norm_kernel, kernels.py:104-145): fp32
 // mean, then fp32 centred biased variance, rstd = 1/sqrt(var + eps),
 // z = (x - mean) * rstd * w + b.  CH = 16-byte chunks per lane.
+//
+// LPR = lanes per row, 64 or 32.  With 32 a wavefront works on two rows at once: for rows of
+// 96 chunks (H = 768 in fp16) every lane then has work in every pass -- with 64 lanes a
+// quarter of them idle in the second pass -- and twice the rows are in flight per wavefront
+// (LayerNorm at the headline: 89 -> 74 us).  The launchers pick 32 when that wastes fewer lanes.
 // ---------------------------------------------------------------------------
-template <typename T, int CH>
+template <typename T, int CH, int LPR>
 __global__ __launch_bounds__(256) void layernorm_vec_kernel(
     const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
     T* __restrict__ out, int64_t M, int H, float eps) {
   typedef typename Vec<T>::type V;
   constexpr int VN = Vec<T>::N;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & (LPR - 1);
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
   if (row >= M) return;
   const int nchunks = H / VN;
   const V* xr = reinterpret_cast<const V*>(x + row * H);
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * LPR;
     if (c < nchunks) {
       V t = __builtin_nontemporal_load(xr + c);
 #pragma unroll
@@ -112,11 +117,11 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
       for (int j = 0; j < VN; ++j) v[i][j] = 0.f;
     }
   }
-  const float mean = wave_sum(s) / (float)H;
+  const float mean = group_sum<LPR>(s) / (float)H;
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    if (lane + i * 64 < nchunks) {
+    if (lane + i * LPR < nchunks) {
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
         const float d = v[i][j] - mean;
@@ -124,14 +129,14 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
       }
     }
   }
-  const float var = wave_sum(q) / (float)H;
+  const float var = group_sum<LPR>(q) / (float)H;
   const float rstd = 1.0f / sqrtf(var + eps);
   const V* wv = reinterpret_cast<const V*>(w);
   const V* bv = reinterpret_cast<const V*>(b);
   V* o = reinterpret_cast<V*>(out + row * H);
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * LPR;
     if (c < nchunks) {
       V tw = wv[c], tb = bv[c], to;
 #pragma unroll
@@ -144,61 +149,6 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
       // instead of HBM ran 12 % faster (its operand loads are only one k-tile ahead)
       o[c] = to;
     }
-  }
-}
-
-// The same for rows of exactly 32 * CH chunks (H = 768: 96 chunks of 8 halves): half a wavefront
-// per row, two rows per wavefront.  Every lane then has work in every chunk (with 64 lanes a
-// quarter of them idle in the second chunk of a 96-chunk row) and a wavefront keeps twice the rows
-// in flight.  Sums run over 32 lanes (shuffle distances 16..1 never leave a half).
-template <typename T, int CH>
-__global__ __launch_bounds__(256) void layernorm_half_kernel(
-    const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
-    T* __restrict__ out, int64_t M, int H, float eps) {
-  typedef typename Vec<T>::type V;
-  constexpr int VN = Vec<T>::N;
-  const int sub = threadIdx.x & 31;
-  const int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-  if (row >= M) return;
-  const V* xr = reinterpret_cast<const V*>(x + row * H);
-  float v[CH][VN];
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    V t = __builtin_nontemporal_load(xr + sub + i * 32);
-#pragma unroll
-    for (int j = 0; j < VN; ++j) {
-      v[i][j] = (float)t[j];
-      s += v[i][j];
-    }
-  }
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
-  const float mean = s / (float)H;
-  float q = 0.f;
-#pragma unroll
-  for (int i = 0; i < CH; ++i)
-#pragma unroll
-    for (int j = 0; j < VN; ++j) {
-      const float d = v[i][j] - mean;
-      q += d * d;
-    }
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, kWave);
-  const float rstd = 1.0f / sqrtf(q / (float)H + eps);
-  const V* wv = reinterpret_cast<const V*>(w);
-  const V* bv = reinterpret_cast<const V*>(b);
-  V* o = reinterpret_cast<V*>(out + row * H);
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int c = sub + i * 32;
-    V tw = wv[c], tb = bv[c], to;
-#pragma unroll
-    for (int j = 0; j < VN; ++j) {
-      const float z = (v[i][j] - mean) * rstd;
-      to[j] = (T)(z * (float)tw[j] + (float)tb[j]);
-    }
-    o[c] = to;  // cached store, as above
   }
 }
 
@@ -230,14 +180,14 @@ __global__ __launch_bounds__(256) void layernorm_scalar_kernel(
 // ---------------------------------------------------------------------------
 // Row softmax: fp32 max, exp(x - max), fp32 sum, divide.
 // ---------------------------------------------------------------------------
-template <typename T, int CH>
+template <typename T, int CH, int LPR>
 __global__ __launch_bounds__(256) void softmax_vec_kernel(const T* __restrict__ x,
                                                           T* __restrict__ out,
                                                           int64_t M, int H) {
   typedef typename Vec<T>::type V;
   constexpr int VN = Vec<T>::N;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & (LPR - 1);
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
   if (row >= M) return;
   const int nchunks = H / VN;
   const V* xr = reinterpret_cast<const V*>(x + row * H);
@@ -245,7 +195,7 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(const T* __restrict__ 
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * LPR;
     if (c < nchunks) {
       V t = __builtin_nontemporal_load(xr + c);
 #pragma unroll
@@ -258,7 +208,7 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(const T* __restrict__ 
       for (int j = 0; j < VN; ++j) v[i][j] = -INFINITY;
     }
   }
-  mx = wave_max(mx);
+  mx = group_max<LPR>(mx);
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
@@ -268,11 +218,11 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(const T* __restrict__ 
       s += v[i][j];
     }
   }
-  const float inv = 1.0f / wave_sum(s);
+  const float inv = 1.0f / group_sum<LPR>(s);
   V* o = reinterpret_cast<V*>(out + row * H);
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * LPR;
     if (c < nchunks) {
       V to;
 #pragma unroll
@@ -342,6 +292,13 @@ __global__ __launch_bounds__(256) void pack_transpose_kernel(const T* __restrict
 // ---------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------
+// Lanes per row for rows of `nchunks` 16-byte chunks: 32 if that leaves fewer idle lane slots
+// than 64 (96 chunks: 3 passes of 32 against 2 passes of 64 with a quarter empty).
+static inline int lanes_per_row(int nchunks) {
+  const int slots32 = (nchunks + 31) / 32 * 32, slots64 = (nchunks + 63) / 64 * 64;
+  return slots32 < slots64 ? 32 : 64;
+}
+
 template <typename T>
 static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
                           void* out, int64_t rows, int64_t L, int H, Dropout drop,
@@ -359,8 +316,12 @@ static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
   const bool aligned = (H % Vec<T>::N) == 0 && ((uintptr_t)wte % 16) == 0 &&
                        ((uintptr_t)wpe % 16) == 0 && ((uintptr_t)out % 16) == 0;
   if (aligned)
-    hipLaunchKernelGGL(embed_vec_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
-                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+    if (lanes_per_row(H / Vec<T>::N) == 32)
+      hipLaunchKernelGGL((embed_vec_kernel<T, 32>), dim3((unsigned)((rows + 7) / 8)), dim3(256), 0,
+                         st, ids, (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+    else
+      hipLaunchKernelGGL((embed_vec_kernel<T, 64>), dim3(grid), dim3(256), 0, st, ids,
+                         (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
   else
     hipLaunchKernelGGL(embed_scalar_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
                        (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
@@ -375,18 +336,15 @@ int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out
 
 template <typename T, int CH>
 static void ln_go(const void* x, const void* w, const void* b, void* out, int64_t M,
-                  int H, float eps, hipStream_t st) {
-  hipLaunchKernelGGL((layernorm_vec_kernel<T, CH>), dim3((unsigned)((M + 3) / 4)),
-                     dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
-                     (T*)out, M, H, eps);
-}
-
-template <typename T, int CH>
-static void ln_half_go(const void* x, const void* w, const void* b, void* out, int64_t M,
-                       int H, float eps, hipStream_t st) {
-  hipLaunchKernelGGL((layernorm_half_kernel<T, CH>), dim3((unsigned)((M + 7) / 8)),
-                     dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
-                     (T*)out, M, H, eps);
+                  int H, float eps, int lpr, hipStream_t st) {
+  if (lpr == 32)
+    hipLaunchKernelGGL((layernorm_vec_kernel<T, CH, 32>), dim3((unsigned)((M + 7) / 8)),
+                       dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
+                       (T*)out, M, H, eps);
+  else
+    hipLaunchKernelGGL((layernorm_vec_kernel<T, CH, 64>), dim3((unsigned)((M + 3) / 4)),
+                       dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
+                       (T*)out, M, H, eps);
 }
 
 template <typename T>
@@ -396,24 +354,15 @@ static int launch_layernorm_t(const void* x, const void* w, const void* b, void*
   const bool aligned = (H % VN) == 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0 &&
                        ((uintptr_t)out % 16) == 0;
-  if (aligned && (H / VN) % 32 == 0) {
-    switch (H / VN / 32) {
-      case 1: ln_half_go<T, 1>(x, w, b, out, M, H, eps, st); return 0;
-      case 2: ln_half_go<T, 2>(x, w, b, out, M, H, eps, st); return 0;
-      case 3: ln_half_go<T, 3>(x, w, b, out, M, H, eps, st); return 0;
-      case 4: ln_half_go<T, 4>(x, w, b, out, M, H, eps, st); return 0;
-      case 6: ln_half_go<T, 6>(x, w, b, out, M, H, eps, st); return 0;
-      default: break;
-    }
-  }
-  const int need = aligned ? (H / VN + 63) / 64 : 1 << 30;
-  if (need <= 1) ln_go<T, 1>(x, w, b, out, M, H, eps, st);
-  else if (need <= 2) ln_go<T, 2>(x, w, b, out, M, H, eps, st);
-  else if (need <= 3) ln_go<T, 3>(x, w, b, out, M, H, eps, st);
-  else if (need <= 4) ln_go<T, 4>(x, w, b, out, M, H, eps, st);
-  else if (need <= 8) ln_go<T, 8>(x, w, b, out, M, H, eps, st);
-  else if (need <= 16) ln_go<T, 16>(x, w, b, out, M, H, eps, st);
-  else if (need <= 32) ln_go<T, 32>(x, w, b, out, M, H, eps, st);
+  const int lpr = lanes_per_row(H / VN);
+  const int need = aligned ? (H / VN + lpr - 1) / lpr : 1 << 30;
+  if (need <= 1) ln_go<T, 1>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 2) ln_go<T, 2>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 3) ln_go<T, 3>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 4) ln_go<T, 4>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 8) ln_go<T, 8>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 16) ln_go<T, 16>(x, w, b, out, M, H, eps, lpr, st);
+  else if (need <= 32) ln_go<T, 32>(x, w, b, out, M, H, eps, lpr, st);
   else
     hipLaunchKernelGGL(layernorm_scalar_kernel<T>, dim3((unsigned)((M + 3) / 4)),
                        dim3(256), 0, st, (const T*)x, (const T*)w, (const T*)b,
@@ -428,9 +377,13 @@ int launch_layernorm(const void* x, const void* w, const void* b, void* out,
 }
 
 template <typename T, int CH>
-static void sm_go(const void* x, void* out, int64_t M, int H, hipStream_t st) {
-  hipLaunchKernelGGL((softmax_vec_kernel<T, CH>), dim3((unsigned)((M + 3) / 4)),
-                     dim3(256), 0, st, (const T*)x, (T*)out, M, H);
+static void sm_go(const void* x, void* out, int64_t M, int H, int lpr, hipStream_t st) {
+  if (lpr == 32)
+    hipLaunchKernelGGL((softmax_vec_kernel<T, CH, 32>), dim3((unsigned)((M + 7) / 8)),
+                       dim3(256), 0, st, (const T*)x, (T*)out, M, H);
+  else
+    hipLaunchKernelGGL((softmax_vec_kernel<T, CH, 64>), dim3((unsigned)((M + 3) / 4)),
+                       dim3(256), 0, st, (const T*)x, (T*)out, M, H);
 }
 
 template <typename T>
@@ -439,14 +392,15 @@ static int launch_softmax_t(const void* x, void* out, int64_t M, int H,
   constexpr int VN = Vec<T>::N;
   const bool aligned =
       (H % VN) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
-  const int need = aligned ? (H / VN + 63) / 64 : 1 << 30;
-  if (need <= 1) sm_go<T, 1>(x, out, M, H, st);
-  else if (need <= 2) sm_go<T, 2>(x, out, M, H, st);
-  else if (need <= 3) sm_go<T, 3>(x, out, M, H, st);
-  else if (need <= 4) sm_go<T, 4>(x, out, M, H, st);
-  else if (need <= 8) sm_go<T, 8>(x, out, M, H, st);
-  else if (need <= 16) sm_go<T, 16>(x, out, M, H, st);
-  else if (need <= 32) sm_go<T, 32>(x, out, M, H, st);
+  const int lpr = lanes_per_row(H / VN);
+  const int need = aligned ? (H / VN + lpr - 1) / lpr : 1 << 30;
+  if (need <= 1) sm_go<T, 1>(x, out, M, H, lpr, st);
+  else if (need <= 2) sm_go<T, 2>(x, out, M, H, lpr, st);
+  else if (need <= 3) sm_go<T, 3>(x, out, M, H, lpr, st);
+  else if (need <= 4) sm_go<T, 4>(x, out, M, H, lpr, st);
+  else if (need <= 8) sm_go<T, 8>(x, out, M, H, lpr, st);
+  else if (need <= 16) sm_go<T, 16>(x, out, M, H, lpr, st);
+  else if (need <= 32) sm_go<T, 32>(x, out, M, H, lpr, st);
   else
     hipLaunchKernelGGL(softmax_scalar_kernel<T>, dim3((unsigned)((M + 3) / 4)),
                        dim3(256), 0, st, (const T*)x, (T*)out, M, H);
