@@ -14,8 +14,9 @@ A step is one forward pass (hidden state [512, 300, 768], like the reference's f
 stops at the final LayerNorm) with the token ids already resident in HBM.  Prints ONE JSON
 line.  Beside the whole-forward numbers it carries
   * "roofline": the dominant kernel (the ffn1 GEMM, M=153600 N=3072 K=768, GELU epilogue) timed
-    live with events around each of its launches inside the timed region; achieved = 2*M*N*K /
-    mean duration against the 2.5 PFLOP/s dense fp16 MFMA peak;
+    live with events around each of its calls inside the timed region (a call is one launch of
+    the persistent kernel plus, at this shape, one of the small-tile kernel for the last 768
+    rows); achieved = 2*M*N*K / mean duration against the 2.5 PFLOP/s dense fp16 MFMA peak;
   * "cpu_baseline": the plain PyTorch fp32 forward of the same architecture (the stand-in for the
     reference's CPU-side comparator, HF GPT2Model in fp32) on this box's host cores, on a
     bounded sample of the same workload.
@@ -43,10 +44,10 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
 }
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
-# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (952.9 MB after scaling by
+# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (999.8 MB after scaling by
 # the copy kernel of --traffic-calibration) + WRITE_SIZE (943.8 MB); the counters cannot be read
 # from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
-FFN1_TRAFFIC_BYTES = 1.897e9
+FFN1_TRAFFIC_BYTES = 1.944e9
 
 
 def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
@@ -279,10 +280,12 @@ def main():
                                        else ", hidden-state output (no LM head)"),
                    "tokens_per_step": tokens, "n_layer": arch["n_layer"], "n_embd": h,
                    "n_head": arch["n_head"]},
-        "roofline": {"kernel": f"ffn1 GEMM (gemm_stream_kernel / gemm_kernel: M={tokens} N={4 * h} K={h}, bias+GELU epilogue)",
+        # one ffn1 call = gemm_stream_kernel on the row tiles that fill whole rounds of the
+        # persistent workgroups + gemm_kernel<128,128> on the rows left over (none for some shapes)
+        "roofline": {"kernel": f"ffn1 GEMM, both launches of a call (gemm_stream_kernel + small-tile gemm_kernel for the last rows: M={tokens} N={4 * h} K={h}, bias+GELU epilogue)",
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16 / 1e12,
                      "unit": "TFLOP/s", "frac": round(achieved * 1e12 / PEAK_FP16, 4),
-                     "avg_ms": round(ffn1_ms, 4), "launches": len(ffn1_events),
+                     "avg_ms": round(ffn1_ms, 4), "calls": len(ffn1_events),
                      "traffic": FFN1_TRAFFIC_BYTES if arch is ARCH and batch == BATCH else None},
     }
     line["cpu_baseline"] = None if (args.no_cpu_baseline or not headline) else cpu_baseline()
