@@ -142,6 +142,9 @@ int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wla
  *   residual [M][N] or NULL     out [M][N]
  * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
  * (may be NULL when that is 0).
+ * Any M, N, K >= 1 and any pointer alignment the element type allows are accepted; the fast
+ * epilogues need N a multiple of 8 (fp16) or 4 (fp32) and 16-byte aligned bias, residual and
+ * out, everything else takes element-wise code with the same results.
  * Dropout (0 < p < 1; 0 = none) sits between the GELU and the residual
  * (kernels.py:245-255): keep where rand(seed, (uint32)(m*N + n)) > p, divide by (1 - p);
  * same generator as gptmi_embed, reference seed 1337 (kernels.py:181).
@@ -160,7 +163,8 @@ int gptmi_linear(const void* x, const void* W, const void* bias,
  * Replaces matmul_and_split_qkv(x, weight, bias, num_heads) -> kernels.py:347-367
  * (fused_ffn followed by split + 3 x view/transpose/contiguous copies).
  *   x [B*L][K]   W [K][3*heads*d] (GPTMI_W_KN) or packed   bias [3*heads*d] or NULL
- *   q, k, v [B][heads][L][d]       d a multiple of 8
+ *   q, k, v [B][heads][L][d]       d a multiple of 8 (GPTMI_ERR_UNSUPPORTED otherwise; the
+ *                                  16-byte scatter stores also need 16-byte aligned q, k, v)
  */
 int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
                      void* k, void* v, int64_t B, int64_t L, int64_t heads,
