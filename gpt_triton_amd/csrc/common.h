@@ -46,10 +46,10 @@ __device__ __forceinline__ float group_max(float v) {
 // that is x * sigmoid(2u) = x / (1 + exp(-2u)); evaluated here as one exp2 and
 // one hardware reciprocal (1 ulp), ~1e-7 relative from the reference's form.
 __device__ __forceinline__ float gelu_new(float x) {
-  // -2 * sqrt(2/pi) * log2(e)
-  const float k = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
-  const float inner = x * fmaf(0.044715f, x * x, 1.0f);
-  const float e = __builtin_amdgcn_exp2f(k * inner);
+  // k = -2 * sqrt(2/pi) * log2(e), folded into the cubic's coefficients: exp(-2u) = exp2(x (k +
+  // 0.044715 k x^2)) -- one multiplication fewer per element of a GELU epilogue
+  constexpr float k = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  const float e = __builtin_amdgcn_exp2f(x * fmaf(0.044715f * k, x * x, k));
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
