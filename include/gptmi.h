@@ -139,7 +139,8 @@ int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wla
  * kernels.py:260-315 and fused_ffn_kernel -> kernels.py:169-257.
  *   x [M][K]   W [K][N] (GPTMI_W_KN), [N][K] (GPTMI_W_NK) or packed (GPTMI_W_PACKED)
  *   bias [N] or NULL
- *   residual [M][N] or NULL     out [M][N]
+ *   residual [M][N] or NULL     out [M][N] (may be the residual's own memory: every
+ *                               element is read before it is written)
  * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
  * (may be NULL when that is 0).
  * Any M, N, K >= 1 and any pointer alignment the element type allows are accepted; the fast

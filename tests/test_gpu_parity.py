@@ -223,6 +223,28 @@ def test_fused_ffn_leading_dims_and_residual_view(K, gpu_device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd", [(2304, 768, 768), (2500, 768, 256), (300, 256, 128)])
+def test_fused_ffn_residual_in_place_and_misaligned(K, gpu_device, dtype, M, N, Kd):
+    """Through the C ABI as a caller that updates its residual stream in place would use it:
+    out aliases residual (every element is read before it is written), and a residual that
+    is only 8-byte aligned (the 16-byte paths must step aside, not fault or misread)."""
+    x, w, b, res = ffn_inputs(M, N, Kd, dtype, seed=11, gaussian=True)
+    want = O.fused_ffn(x, w, bias=b, residual=res)
+    xd, wd, bd = dev(x, gpu_device), dev(w, gpu_device), dev(b, gpu_device)
+    z = dev(res, gpu_device).clone()
+    K._linear(xd, wd, bd, z, z, False, 0.0, K._lib.GPTMI_W_KN, "in place")
+    check(host(z), want, dtype, "ffn in place")
+    shift = 8 // z.element_size()  # elements in 8 bytes
+    buf = torch.empty(M * N + shift, device=gpu_device, dtype=dtype)
+    r8 = buf[shift:].view(M, N)
+    assert r8.data_ptr() % 16 == 8
+    r8.copy_(dev(res, gpu_device))
+    z = torch.empty((M, N), device=gpu_device, dtype=dtype)
+    K._linear(xd, wd, bd, r8, z, False, 0.0, K._lib.GPTMI_W_KN, "misaligned residual")
+    check(host(z), want, dtype, "ffn misaligned residual")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_lm_head_transposed_weight(K, gpu_device, dtype):
     r = np.random.default_rng(21)
     x = r.standard_normal((130, 768)).astype(NP[dtype])
