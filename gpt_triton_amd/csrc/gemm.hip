@@ -23,15 +23,22 @@
 //   * each wavefront owns a (BM/WM) x (BN/WN) sub-tile as 32x32 MFMA blocks.
 //     The MFMA is issued as D[n][m] (weight rows as the first operand) so a
 //     lane ends up with 4 consecutive n for one m;
-//   * the epilogue applies bias/GELU in that layout, stages fp32 through LDS
-//     and stores row-major runs (see store_wave_tile);
+//   * the epilogue applies bias/GELU in that layout, transposes through a wavefront-private
+//     LDS slab and stores row-major runs.  Four forms (dispatch in store_wave_tile and at the
+//     end of the kernels): fp16 output, whole tile, no residual -> rounded first, slab of halves,
+//     16-byte stores (store_wave_tile_h); the same with a residual -> the residual tile is
+//     brought into the operand stages by direct loads as these fall free and added in the
+//     accumulator layout before the one rounding (store_wave_tile_rl); everything else that is a
+//     whole tile with aligned pointers -> fp32 slab, 8- or 16-byte accesses (store_wave_tile_v
+//     FAST); tiles on the matrix edge, odd N, unaligned pointers, dropout -> the same slab with
+//     element-wise predicated accesses;
 //   * workgroup ids are remapped so each XCD (ids are dealt round-robin over
 //     the 8 XCDs) gets a contiguous range of tiles; inside a group of column tiles whose
 //     weight panels fit the XCD's L2 the column runs fastest, so the tiles that share a row
 //     block of A run on the same L2 at the same time.
 // gemm_stream_kernel (further down) is the persistent form of the 256 x 256 x 64 configuration
-// for whole-tile shapes: one workgroup per CU walks tiles and the pipeline runs across tile
-// boundaries.
+// for whole-tile shapes without residual: one workgroup per CU walks tiles and the pipeline
+// runs across tile boundaries.  launch_shape (at the end) picks kernel and configuration.
 #include "common.h"
 #include "launch.h"
 
