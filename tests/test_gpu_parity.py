@@ -559,6 +559,26 @@ def test_full_size_qkv_split(K, gpu_device):
         check(got[idx].cpu().numpy(), want, torch.float16, f"qkv full size {name}")
 
 
+def test_full_size_forward_sampled_sequences(gpu_device):
+    """BASELINE config 3: the whole 124M forward in fp16 at batch 512 x seqlen 300 -- the shapes
+    at which the persistent GEMM kernels, their small-tile tails and the resident attention
+    kernel run.  Sequences do not interact, so a few of them (first, middle, both sides of the
+    row where the GEMM launches are split, last) are compared with the oracle run on those
+    sequences alone; tolerance as for the small models, 2e-2 absolute."""
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig
+
+    cfg = dict(n_layer=12, n_head=12, n_embd=768, vocab_size=50257, block_size=1024)
+    params = O.synthetic_params(**cfg, seed=1337, dtype=np.float16)
+    ids = O.synthetic_ids(512, 300, cfg["vocab_size"], seed=1337)
+    model = load_params(FusedGPT(GPTConfig(dropout=0.1, **cfg)), params, torch.float16, gpu_device)
+    hidden = model(dev(ids, gpu_device))
+    assert hidden.shape == (512, 300, 768) and torch.isfinite(hidden).all()
+    seqs = [0, 255, 509, 510, 511]
+    want = O.gpt2_forward(params, ids[seqs], cfg["n_head"])
+    got = hidden[torch.tensor(seqs, device=gpu_device)].cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= 2e-2
+
+
 def test_full_size_attention_heads(K, gpu_device):
     """BASELINE config 2: q, k, v [512, 12, 300, 64] fp16; (batch, head) pairs are independent."""
     g = torch.Generator(device="cpu").manual_seed(2)
