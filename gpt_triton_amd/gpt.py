@@ -22,7 +22,7 @@ import torch
 import torch.nn as nn
 
 from .kernels import (flash_attention_v1, fused_embeddings, fused_ffn, fused_layer_norm, lm_head,
-                      matmul_and_split_qkv, pack_weight)
+                      matmul_and_split_qkv, pack_lm_head, pack_weight)
 
 # dense fp16/bf16 tensor throughput, FLOP/s
 GPU_TO_FLOPS = {
@@ -42,11 +42,11 @@ class _PackedWeights:
     def __init__(self):
         self._entries = {}
 
-    def get(self, name, param):
+    def get(self, name, param, pack=pack_weight):
         key = (param.data_ptr(), param._version, param.dtype, tuple(param.shape))
         hit = self._entries.get(name)
         if hit is None or hit[0] != key:
-            hit = (key, pack_weight(param.data))
+            hit = (key, pack(param.data))
             self._entries[name] = hit
         return hit[1]
 
@@ -175,6 +175,19 @@ class FusedGPT(nn.Module):
         ])
         self.layer_norm_weight = nn.Parameter(torch.ones((h,)))
         self.layer_norm_bias = nn.Parameter(torch.zeros((h,)))
+        self._packed = _PackedWeights()
+
+    def train(self, mode=True):
+        self._packed.clear()
+        return super().train(mode)
+
+    def _lm_head_weight(self):
+        # A vocabulary that is not a multiple of 8 (GPT-2's 50257) gets a zero-padded packed image
+        # in eval mode, so that the logits' rows are whole 16-byte units; see kernels.pack_lm_head.
+        w = self.wte_weight
+        if self.training or w.shape[0] % 8 == 0:
+            return w.data
+        return self._packed.get("lm_head", w, pack_lm_head)
 
     def forward(self, x, return_logits=False):
         # causal by construction; no attention or padding mask is taken
@@ -184,7 +197,7 @@ class FusedGPT(nn.Module):
             x = block(x)
         x = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
         if return_logits:
-            return x, lm_head(x, self.wte_weight.data)
+            return x, lm_head(x, self._lm_head_weight())
         return x
 
     def get_fwd_flops(self, num_tokens):

@@ -64,10 +64,11 @@ class PackedWeight:
     """The fp16 [N][round_up(K, 64)] image of a [K, N] weight (see gptmi_pack_weight).  `shape`
     and `dtype` are those of the weight it was made from, so it can stand in for it."""
 
-    __slots__ = ("data", "shape", "dtype", "device")
+    __slots__ = ("data", "shape", "dtype", "device", "vocab")
 
-    def __init__(self, data, shape, dtype):
+    def __init__(self, data, shape, dtype, vocab=None):
         self.data, self.shape, self.dtype, self.device = data, tuple(shape), dtype, data.device
+        self.vocab = vocab  # pack_lm_head: rows of wte before the zero padding
 
     def is_contiguous(self):
         return True
@@ -90,6 +91,25 @@ def pack_weight(weight):
                                    _dtype_code(weight, "pack_weight"), _stream())
     _lib.check(rc, "pack_weight")
     return PackedWeight(buf, weight.shape, weight.dtype)
+
+
+@torch.no_grad()
+def pack_lm_head(wte):
+    """Packs wte [V, H] once for `lm_head`, with the vocabulary padded to a multiple of 8 by zero
+    rows.  GPT-2's V = 50257 is odd: rows of a dense [T, V] fp16 matrix then start on 2-byte
+    boundaries and every logit is stored on its own.  With the padded image the GEMM writes
+    [T, Vp] rows of whole 16-byte units and `lm_head` returns the [.., :V] view of it."""
+    assert wte.dim() == 2 and wte.is_contiguous()
+    dev = _on_gpu(wte)
+    V, H = wte.shape
+    Vp = -(-V // 8) * 8
+    lib = _lib.load()
+    buf = torch.zeros(lib.gptmi_packed_weight_bytes(Vp, H), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_pack_weight(wte.data_ptr(), buf.data_ptr(), V, H, _lib.GPTMI_W_NK,
+                                   _dtype_code(wte, "pack_lm_head"), _stream())
+    _lib.check(rc, "pack_lm_head")
+    return PackedWeight(buf, (H, Vp), wte.dtype, vocab=V)
 
 
 def _wlayout(weight, default):
@@ -205,11 +225,19 @@ def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False, dropout_prob=
 
 @torch.no_grad()
 def lm_head(x, wte):
-    """x @ wte^T for wte [V, H]: logits [*, V] without materialising the transposed weight."""
+    """x @ wte^T: logits [*, V].  `wte` is the [V, H] embedding matrix itself (read in place, no
+    transposed copy; the result is contiguous) or its `pack_lm_head` image (the result is then
+    the [*, :V] view of a buffer whose rows are padded to a multiple of 8 logits)."""
     out_shape_0 = x.shape[:-1]
     x = x.view((-1, x.shape[-1]))
     assert x.is_contiguous()
     assert wte.is_contiguous()
+    if isinstance(wte, PackedWeight):
+        assert wte.vocab is not None and x.shape[1] == wte.shape[0]
+        dev = _on_gpu(x, wte)
+        z = torch.empty((x.shape[0], wte.shape[1]), device=dev, dtype=x.dtype)
+        _linear(x, wte, None, None, z, False, 0.0, _lib.GPTMI_W_PACKED, "lm_head")
+        return z.view((*out_shape_0, wte.shape[1]))[..., :wte.vocab]
     assert x.shape[1] == wte.shape[1]
     dev = _on_gpu(x, wte)
     z = torch.empty((x.shape[0], wte.shape[0]), device=dev, dtype=x.dtype)
