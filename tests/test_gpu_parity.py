@@ -486,6 +486,27 @@ def test_convert_hf_and_load_model_from_local_directory(gpu_device, dtype, tmp_p
     assert np.abs(got - want).max() <= (1e-2 if dtype == torch.float32 else 3e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_forward_captured_in_a_graph(gpu_device, dtype):
+    """The whole forward captured into a HIP graph (gpt.GraphedForward) and replayed with new
+    token ids: every replay, with eager forwards and synchronisations in between, must equal
+    the eager result bit for bit -- the library allocates nothing and keeps no per-call state."""
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig, GraphedForward
+
+    cfg = dict(n_layer=3, n_head=4, n_embd=256, vocab_size=1000, block_size=128)
+    params = O.synthetic_params(**cfg, seed=5, std=0.05, dtype=NP[dtype])
+    model = load_params(FusedGPT(GPTConfig(dropout=0.1, **cfg)), params, dtype, gpu_device)
+    ids = dev(O.synthetic_ids(3, 100, cfg["vocab_size"], seed=5), gpu_device)
+    graphed = GraphedForward(model, ids, return_logits=True)
+    for seed in (6, 7, 8, 9):
+        ids = dev(O.synthetic_ids(3, 100, cfg["vocab_size"], seed=seed), gpu_device)
+        hidden, logits = graphed(ids)
+        torch.cuda.synchronize()
+        want_h, want_l = model(ids, return_logits=True)
+        torch.cuda.synchronize()
+        assert torch.equal(hidden, want_h) and torch.equal(logits, want_l)
+
+
 def test_gpt2_layerwise_fp32(K, gpu_device):
     """Every operator of a 3-layer model, each fed the ORACLE's intermediate activations, so
     that no upstream difference is carried along: fp32 storage, tolerance 1e-5 * max|b| (the
