@@ -3,7 +3,7 @@ comparator, HuggingFace GPT2Model run eagerly in fp32 (bench.py:42-49, test.py:1
 files and weights cannot travel to the GPU box.  Same block order as HF GPT-2
 (ln_1 -> attention -> +residual -> ln_2 -> MLP -> +residual -> ln_f), true fp32 products.
 
-TEST / BASELINE INFRASTRUCTURE ONLY: used by bench.py's cpu_baseline leg and by tests; the
+TEST / CPU-BASELINE INFRASTRUCTURE ONLY: used by bench.py's cpu_baseline leg and by tests; the
 product never imports it.
 """
 import math

@@ -1,6 +1,6 @@
 """GPU parity: every operator of gpt_triton_amd.kernels (through ctypes -> libgptmi.so) against
 the CPU oracle on the same seeded inputs.  Shapes follow the reference's test.py grids plus
-the GPT-2 sizes; the full BASELINE sizes are checked on sub-samples of independent rows/heads.
+the GPT-2 sizes; the full benchmark sizes are checked on sub-samples of independent rows/heads.
 
 Tolerances (stated once, used everywhere):
   * embedding gather: bit exact;
@@ -202,7 +202,7 @@ def test_fused_ffn_gpt2_shapes(K, gpu_device, dtype, M, N, Kd, gelu, use_res):
 
 
 def test_fused_ffn_xl_shapes(K, gpu_device):
-    """BASELINE config 4 widths (d_model 1600, 25 heads, FFN 6400): N = 4800 / 1600 / 6400 are
+    """Benchmark configuration 4 widths (d_model 1600, 25 heads, FFN 6400): N = 4800 / 1600 / 6400 are
     not multiples of the 256-wide tile, K = 1600 / 6400 are multiples of 32 only."""
     for (M, N, Kd, gelu, use_res) in [(2304, 4800, 1600, False, False), (2304, 6400, 1600, True, False),
                                       (2304, 1600, 6400, False, True)]:
@@ -382,7 +382,7 @@ def test_flash_attention_small_heads(K, gpu_device, dtype, D):
 
 
 def test_flash_attention_xl_sequence(K, gpu_device):
-    """BASELINE config 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
+    """Benchmark configuration 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
     K/V do not fit the resident variant)."""
     q, k, v = attn_inputs(1, 5, 1024, 64, torch.float16, gaussian=True, seed=11)
     z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
@@ -447,7 +447,7 @@ def test_gpt2_small_forward(gpu_device, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_gpt2_124m_config0(gpu_device, dtype):
-    """BASELINE config 0: 12 x 768 x 12 heads, vocab 50257, 1024 positions, N(0, 0.02)
+    """Benchmark configuration 0: 12 x 768 x 12 heads, vocab 50257, 1024 positions, N(0, 0.02)
     weights, batch 2 x seqlen 64; hidden state and logits [2, 64, 50257]."""
     from gpt_triton_amd.gpt import FusedGPT, GPTConfig
 
@@ -550,9 +550,9 @@ def test_gpt2_layerwise_fp32(K, gpu_device):
               x, f"layer {i} ffn2")
 
 
-# ----------------------------------------------------------------------------- BASELINE sizes
+# ----------------------------------------------------------------------------- benchmark sizes
 def test_full_size_ffn_rows(K, gpu_device):
-    """BASELINE config 1: X [153600, 768] fp16 @ W [768, 3072] + b -> GELU, then the down
+    """Benchmark configuration 1: X [153600, 768] fp16 @ W [768, 3072] + b -> GELU, then the down
     projection [153600, 3072] @ [3072, 768] + b (+ residual).  Rows of a GEMM are independent,
     so a random sample of rows is compared with the oracle run on those rows alone."""
     g = torch.Generator(device="cpu").manual_seed(1)
@@ -602,7 +602,7 @@ def test_full_size_qkv_split(K, gpu_device):
 
 
 def test_full_size_forward_sampled_sequences(gpu_device):
-    """BASELINE config 3: the whole 124M forward in fp16 at batch 512 x seqlen 300 -- the shapes
+    """Benchmark configuration 3: the whole 124M forward in fp16 at batch 512 x seqlen 300 -- the shapes
     at which the persistent GEMM kernels, their small-tile tails and the resident attention
     kernel run.  Sequences do not interact, so a few of them (first, middle, both sides of the
     row where the GEMM launches are split, last) are compared with the oracle run on those
@@ -622,7 +622,7 @@ def test_full_size_forward_sampled_sequences(gpu_device):
 
 
 def test_full_size_attention_heads(K, gpu_device):
-    """BASELINE config 2: q, k, v [512, 12, 300, 64] fp16; (batch, head) pairs are independent."""
+    """Benchmark configuration 2: q, k, v [512, 12, 300, 64] fp16; (batch, head) pairs are independent."""
     g = torch.Generator(device="cpu").manual_seed(2)
     B, N, L, D = 512, 12, 300, 64
     q, k, v = (torch.randn((B, N, L, D), generator=g).half() for _ in range(3))
@@ -637,7 +637,7 @@ def test_full_size_attention_heads(K, gpu_device):
 
 
 def test_full_size_rowops(K, gpu_device):
-    """BASELINE config 2: LayerNorm and softmax on [153600, 768] fp16."""
+    """Benchmark configuration 2: LayerNorm and softmax on [153600, 768] fp16."""
     g = torch.Generator(device="cpu").manual_seed(3)
     M, H = 153600, 768
     x = torch.randn((M, H), generator=g).half()
