@@ -578,7 +578,8 @@ def test_full_size_ffn_rows(K, gpu_device):
     assert (y.float().abs().sum(dim=1) > 0).all()
 
 
-def test_full_size_qkv_split(K, gpu_device):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_full_size_qkv_split(K, gpu_device, dtype):
     """The headline qkv product: [512, 300, 768] fp16 @ [768, 2304] + b, scattered to q, k, v
     [512, 12, 300, 64].  600 x 9 tiles are 21 rounds of 256 workgroups and 24 tiles more, so
     the launcher sends the last 768 token rows to the small-tile kernel with a row offset:
@@ -587,9 +588,9 @@ def test_full_size_qkv_split(K, gpu_device):
     g = torch.Generator(device="cpu").manual_seed(3)
     B, L, heads, d = 512, 300, 12, 64
     h = heads * d
-    x = torch.randn((B, L, h), generator=g).half()
-    w = (0.03 * torch.randn((h, 3 * h), generator=g)).half()
-    b = (0.1 * torch.randn(3 * h, generator=g)).half()
+    x = torch.randn((B, L, h), generator=g).to(dtype)
+    w = (0.03 * torch.randn((h, 3 * h), generator=g)).to(dtype)
+    b = (0.1 * torch.randn(3 * h, generator=g)).to(dtype)
     q, k, v = K.matmul_and_split_qkv(x.to(gpu_device), w.to(gpu_device), b.to(gpu_device), heads)
     assert q.shape == (B, heads, L, d) and q.is_contiguous()
     for t in (q, k, v):
@@ -598,7 +599,7 @@ def test_full_size_qkv_split(K, gpu_device):
     wq, wk, wv = O.matmul_and_split_qkv(x[seqs].numpy(), w.numpy(), b.numpy(), heads)
     idx = torch.tensor(seqs, device=gpu_device)
     for got, want, name in ((q, wq, "q"), (k, wk, "k"), (v, wv, "v")):
-        check(got[idx].cpu().numpy(), want, torch.float16, f"qkv full size {name}")
+        check(got[idx].cpu().numpy(), want, dtype, f"qkv full size {name}")
 
 
 def test_full_size_forward_sampled_sequences(gpu_device):
