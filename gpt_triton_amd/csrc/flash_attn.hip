@@ -68,8 +68,11 @@ __device__ __forceinline__ h8 zero_h8() {
 // D = head size.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
 // position c ^ (r&7)) and V^T tile [D][64] (8-byte unit u of row d at position
 // u ^ ((d>>1)&15)).
+#ifndef GPTMI_TILED_WAVES
+#define GPTMI_TILED_WAVES 2
+#endif
 template <int D, typename T, bool BLND, bool DROP>
-__global__ __launch_bounds__(256) void flash_attn_kernel(
+__global__ __launch_bounds__(256, (D == 64 && !DROP) ? GPTMI_TILED_WAVES : 1) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     T* __restrict__ O, int heads, int L, float scale, DropoutArgs drop) {
   constexpr int CH = D / 8;             // 16-byte chunks per row
@@ -131,26 +134,29 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
       scol[i] = (s >> 4) * 8;
     }
   }
-  h8 stg[NLD];
+  // Two register sets: tile u travels in set u % 2.  It is requested two steps before it is
+  // multiplied (during step u - 2) and written to LDS at the end of step u - 1, so a global load
+  // has a whole step of arithmetic plus a barrier to arrive, not a fraction of one.
+  h8 stg[2][NLD];
 
-  auto load_tile = [&](int t) {
+  auto load_tile = [&](int t, h8 (&dst)[NLD]) {
     const int k0 = t * BKEY;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       int row = k0 + srow[i];
       row = row < L ? row : L - 1;
-      stg[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
+      dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
     }
   };
 
-  auto store_tile = [&](int stage) {
+  auto store_tile = [&](int stage, const h8 (&src)[NLD]) {
     char* ks_ = smem + stage * STAGE;
     char* vs_ = ks_ + K_BYTES;
     if (role_k) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         const int key = srow[i], c = scol[i] >> 3;
-        *reinterpret_cast<h8*>(ks_ + key * (D * 2) + ((c ^ (key & 7)) << 4)) = stg[i];
+        *reinterpret_cast<h8*>(ks_ + key * (D * 2) + ((c ^ (key & 7)) << 4)) = src[i];
       }
     } else {
 #pragma unroll
@@ -159,7 +165,7 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int d = d0 + j;
-          h4 col = {stg[4 * u][j], stg[4 * u + 1][j], stg[4 * u + 2][j], stg[4 * u + 3][j]};
+          h4 col = {src[4 * u][j], src[4 * u + 1][j], src[4 * u + 2][j], src[4 * u + 3][j]};
           *reinterpret_cast<h4*>(vs_ + d * 128 + ((kg ^ ((d >> 1) & 15)) << 3)) = col;
         }
       }
@@ -173,12 +179,16 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
   float mrun = -INFINITY, den = 0.f;
 
-  load_tile(0);
-  store_tile(0);
+  load_tile(0, stg[0]);
+  if (nt > 1) load_tile(1, stg[1]);
+  store_tile(0, stg[0]);
   __syncthreads();
 
-  for (int t = 0; t < nt; ++t) {
-    if (t + 1 < nt) load_tile(t + 1);
+  // one step = one key tile; `step` is instantiated for even and odd t so that the register
+  // set of tile t + 1 (written to LDS at the end) and of tile t + 2 (requested at the start,
+  // into the set tile t just left) are compile-time choices
+  auto step = [&](int t, h8 (&set_same)[NLD], h8 (&set_next)[NLD]) {
+    if (t + 2 < nt) load_tile(t + 2, set_same);
     const int k0 = t * BKEY;
     if (wave_active && k0 <= qw0 + 31) {
       const char* ks_ = smem + (t & 1) * STAGE;
@@ -199,34 +209,62 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
       }
       // ---- scale, causal mask, running max -----------------------------------
       const bool need_mask = k0 + BKEY - 1 > qw0;
-      float bmax = -INFINITY;
+      if (need_mask) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float x = s[kb][r] * scale;
-          if (need_mask) {
+          for (int r = 0; r < 16; ++r) {
             const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-            x = key <= q ? x : -INFINITY;
+            s[kb][r] = key <= q ? s[kb][r] : -INFINITY;
           }
-          s[kb][r] = x;
-          bmax = fmaxf(bmax, x);
-        }
-      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
-      const float mnew = bmax > mrun ? bmax : mrun;
-      const float mult = softmax_exp<T>(mrun - mnew);
-      float psum = 0.f;
+      }
+      float mult, psum = 0.f;
+      if constexpr (sizeof(T) == 2 && !DROP) {
+        // fp16 storage: running max on the raw scores, scale * log2(e) folded into one fused
+        // multiply-add in front of exp2 (as in the resident kernel below)
+        const float c = scale * 1.4426950408889634f;
+        float bmax = -INFINITY;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float p = softmax_exp<T>(s[kb][r] - mnew);
-          s[kb][r] = p;
-          psum += p;
-        }
+          for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, s[kb][r]);
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+        const float mnew = bmax > mrun ? bmax : mrun;
+        mult = __builtin_amdgcn_exp2f((mrun - mnew) * c);
+        const float m2 = mnew * c;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][r], c, -m2));
+            s[kb][r] = p;
+            psum += p;
+          }
+        mrun = mnew;
+      } else {
+        float bmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            s[kb][r] *= scale;
+            bmax = fmaxf(bmax, s[kb][r]);
+          }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+        const float mnew = bmax > mrun ? bmax : mrun;
+        mult = softmax_exp<T>(mrun - mnew);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = softmax_exp<T>(s[kb][r] - mnew);
+            s[kb][r] = p;
+            psum += p;
+          }
+        mrun = mnew;
+      }
       psum += __shfl_xor(psum, 32, kWave);
       den = den * mult + psum;
-      mrun = mnew;
       if constexpr (DROP) {
         // dropout of P after the denominator has summed it, before the fp16 rounding;
         // offset = query * L + key, the same for every batch and head (kernels.py:457-460)
@@ -269,8 +307,12 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(
           }
         }
     }
-    if (t + 1 < nt) store_tile((t + 1) & 1);
+    if (t + 1 < nt) store_tile((t + 1) & 1, set_next);
     __syncthreads();
+  };
+  for (int t = 0; t < nt; t += 2) {
+    step(t, stg[0], stg[1]);
+    if (t + 1 < nt) step(t + 1, stg[1], stg[0]);
   }
 
   // ---- out[q][d] = O^T[d][q] / den ------------------------------------------
