@@ -384,7 +384,7 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
   //   V unit  u -> d-chunk u % CH, key group u / CH (4 keys); keys past the end repeat the
   //   last row: their weights are exactly 0
   constexpr int NT = NW * 64;
-  constexpr int KI = 2560 / NT, VI = (640 + NT - 1) / NT;
+  constexpr int KI = (2560 + NT - 1) / NT, VI = (640 + NT - 1) / NT;
   const int kchunks = L * CH, units = (Lp / 4) * CH;
   h8 kr[KI], vr[VI][4];
 #pragma unroll
