@@ -100,13 +100,20 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
   if (row >= M) return;
   const int nchunks = H / VN;
   const V* xr = reinterpret_cast<const V*>(x + row * H);
+  const V* wv = reinterpret_cast<const V*>(w);
+  const V* bv = reinterpret_cast<const V*>(b);
   float v[CH][VN];
+  V tw[CH], tb[CH];  // weight and bias chunks, requested with the row: off the tail of the row
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     const int c = lane + i * LPR;
     if (c < nchunks) {
       V t = __builtin_nontemporal_load(xr + c);
+      if (CH <= 4) {
+        tw[i] = wv[c];
+        tb[i] = bv[c];
+      }
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
         v[i][j] = (float)t[j];
@@ -131,18 +138,20 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
   }
   const float var = group_sum<LPR>(q) / (float)H;
   const float rstd = 1.0f / sqrtf(var + eps);
-  const V* wv = reinterpret_cast<const V*>(w);
-  const V* bv = reinterpret_cast<const V*>(b);
   V* o = reinterpret_cast<V*>(out + row * H);
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     const int c = lane + i * LPR;
     if (c < nchunks) {
-      V tw = wv[c], tb = bv[c], to;
+      if (CH > 4) {  // long rows: too many registers to hold them from the start
+        tw[i] = wv[c];
+        tb[i] = bv[c];
+      }
+      V to;
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
         const float z = (v[i][j] - mean) * rstd;
-        to[j] = (T)(z * (float)tw[j] + (float)tb[j]);
+        to[j] = (T)(z * (float)tw[i][j] + (float)tb[i][j]);
       }
       // cached (not streaming) store: the [T, H] output is what the following GEMM reads, two
       // or three times over; it fits the 256 MB memory-side cache, and a GEMM fed from there
