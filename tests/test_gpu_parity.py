@@ -244,6 +244,38 @@ def test_fused_ffn_residual_in_place_and_misaligned(K, gpu_device, dtype, M, N, 
     check(host(z), want, dtype, "ffn misaligned residual")
 
 
+def test_fused_ffn_random_shapes(K, gpu_device):
+    """48 seeded random problems across the kernel-selection boundaries: M below and above the
+    big-tile threshold and with ragged last tiles, N odd / a multiple of 4, 8, 64, 256 (which
+    decides the epilogue form), K from 1 to 1100, every combination of bias, GELU and residual,
+    both storage types.  The checker is the same arithmetic in fp32 on the GPU (torch matmul of
+    the fp16-rounded operands), which is quick at these sizes; tolerance as in `check`."""
+    g = torch.Generator(device="cpu").manual_seed(4242)
+    gelu_ref = lambda t: torch.nn.functional.gelu(t, approximate="tanh")
+    for case in range(48):
+        r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+        M = [r(1, 300), r(2048, 2400), r(2500, 5200), 256 * r(8, 20)][case % 4]
+        N = [r(1, 700) | 1, 4 * r(1, 300), 8 * r(1, 200), 64 * r(1, 24), 256 * r(1, 8)][case % 5]
+        Kd = [r(1, 63), 64 * r(1, 16), r(65, 1100)][case % 3]
+        dtype = torch.float16 if case % 2 == 0 else torch.float32
+        bias, gelu, res = bool(case & 1), bool(case & 2), bool(case & 4)
+        x = torch.randn((M, Kd), generator=g).to(dtype)
+        w = (torch.randn((Kd, N), generator=g) / max(1.0, Kd ** 0.5)).to(dtype)
+        b = torch.randn(N, generator=g).to(dtype) if bias else None
+        rs = torch.randn((M, N), generator=g).to(dtype) if res else None
+        D = lambda t: None if t is None else t.to(gpu_device)
+        z = K.fused_ffn(D(x), D(w), bias=D(b), residual=D(rs), add_gelu=gelu)
+        want = D(x).half().float() @ D(w).half().float()
+        if bias:
+            want = want + D(b).float()
+        if gelu:
+            want = gelu_ref(want)
+        if res:
+            want = want + D(rs).float()
+        check(host(z), want.cpu().numpy(), dtype,
+              f"case {case}: M={M} N={N} K={Kd} {dtype} bias={bias} gelu={gelu} res={res}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_lm_head_transposed_weight(K, gpu_device, dtype):
     r = np.random.default_rng(21)
