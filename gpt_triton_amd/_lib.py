@@ -26,6 +26,9 @@ SIGNATURES = {
     "gptmi_pack_weight": (_int, [_vp, _vp, _i64, _i64, _int, _int, _vp]),
     "gptmi_linear": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _f32, _u64, _int,
                             _vp, _sz, _int, _vp]),
+    "gptmi_linear_static_capacity": (_sz, []),
+    "gptmi_linear_static": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _f32, _u64,
+                                   _int, _int, _vp]),
     "gptmi_linear_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                 _vp, _sz, _int, _vp]),
     "gptmi_flash_attn": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _f32,

@@ -5,6 +5,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "common.h"
 #include "launch.h"
 
@@ -89,6 +91,86 @@ static int prepare_operands(const void* x, const void* W, int64_t M, int64_t N, 
     *A = x;
   }
   *Kp = p.Kp;
+  return GPTMI_OK;
+}
+
+// Scratch of gptmi_linear_static: the packed operand images that gptmi_linear puts into the
+// caller's workspace.  Every GPU the library runs on holds its own copy of the array (at its own
+// address) until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress -- never a device address -- so all uses go through static_scratch().
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[GPTMI_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device, resolved once per device; nullptr (and
+// the error text set) on failure.
+static void* static_scratch() {
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("linear_static: cannot identify the current device (%s, device %d)",
+              hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("linear_static: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                hipGetErrorString(e));
+      return nullptr;
+    }
+    ptrs[dev] = p;
+  }
+  return ptrs[dev];
+}
+
+// gptmi_linear and gptmi_linear_static behind their argument checks: pack the operands into
+// `workspace` as the plan says, then the GEMM.
+static int linear_impl(const void* x, const void* W, const void* bias, const void* residual,
+                       void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
+                       uint64_t seed, int wlayout, void* workspace, size_t workspace_bytes,
+                       int dtype, hipStream_t st) {
+  const void *A, *Bt;
+  int Kp;
+  int rc = prepare_operands(x, W, M, N, K, dtype, wlayout, workspace, workspace_bytes, st,
+                            &A, &Bt, &Kp);
+  if (rc) return rc;
+  if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) {
+    set_error("linear: x and W must be 16-byte aligned");
+    return GPTMI_ERR_INVALID;
+  }
+  GemmEpilogue ep = {};
+  ep.bias = bias;
+  ep.residual = residual;
+  ep.out = out;
+  ep.gelu = gelu ? 1 : 0;
+  ep.drop = Dropout{p, seed};
+  ep.qkv = false;
+  ep.f16 = dtype == GPTMI_F16;
+  rc = launch_gemm(A, Bt, M, (int)N, Kp, ep, st);
+  if (rc) return rc;
+  return check_launch("linear");
+}
+
+static int check_linear_args(const void* x, const void* W, const void* out, int64_t M, int64_t N,
+                             int64_t K, float p, int wlayout, int dtype) {
+  if (!x || !W || !out || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
+      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK && wlayout != GPTMI_W_PACKED)) {
+    set_error("linear: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (N > (1 << 30) || K > (1 << 30)) {
+    set_error("linear: N or K too large");
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (!dropout_ok(p)) {
+    set_error("linear: dropout probability %g outside [0, 1)", (double)p);
+    return GPTMI_ERR_INVALID;
+  }
   return GPTMI_OK;
 }
 
@@ -188,40 +270,35 @@ int gptmi_linear(const void* x, const void* W, const void* bias, const void* res
                  void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
                  uint64_t seed, int wlayout, void* workspace, size_t workspace_bytes,
                  int dtype, void* stream) {
-  if (!x || !W || !out || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) ||
-      (wlayout != GPTMI_W_KN && wlayout != GPTMI_W_NK && wlayout != GPTMI_W_PACKED)) {
-    set_error("linear: invalid argument");
-    return GPTMI_ERR_INVALID;
-  }
-  if (N > (1 << 30) || K > (1 << 30)) {
-    set_error("linear: N or K too large");
-    return GPTMI_ERR_UNSUPPORTED;
-  }
-  if (!dropout_ok(p)) {
-    set_error("linear: dropout probability %g outside [0, 1)", (double)p);
-    return GPTMI_ERR_INVALID;
-  }
-  hipStream_t st = (hipStream_t)stream;
-  const void *A, *Bt;
-  int Kp;
-  int rc = prepare_operands(x, W, M, N, K, dtype, wlayout, workspace, workspace_bytes, st,
-                            &A, &Bt, &Kp);
+  const int rc = check_linear_args(x, W, out, M, N, K, p, wlayout, dtype);
   if (rc) return rc;
-  if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) {
-    set_error("linear: x and W must be 16-byte aligned");
-    return GPTMI_ERR_INVALID;
-  }
-  GemmEpilogue ep = {};
-  ep.bias = bias;
-  ep.residual = residual;
-  ep.out = out;
-  ep.gelu = gelu ? 1 : 0;
-  ep.drop = Dropout{p, seed};
-  ep.qkv = false;
-  ep.f16 = dtype == GPTMI_F16;
-  rc = launch_gemm(A, Bt, M, (int)N, Kp, ep, st);
+  return linear_impl(x, W, bias, residual, out, M, N, K, gelu, p, seed, wlayout, workspace,
+                     workspace_bytes, dtype, (hipStream_t)stream);
+}
+
+size_t gptmi_linear_static_capacity(void) { return GPTMI_STATIC_SCRATCH_BYTES; }
+
+int gptmi_linear_static(const void* x, const void* W, const void* bias, const void* residual,
+                        void* out, int64_t M, int64_t N, int64_t K, int gelu, float p,
+                        uint64_t seed, int wlayout, int dtype, void* stream) {
+  const int rc = check_linear_args(x, W, out, M, N, K, p, wlayout, dtype);
   if (rc) return rc;
-  return check_launch("linear");
+  // the size check comes before anything touches the device
+  const size_t need = plan_linear(M, N, K, dtype, wlayout).total;
+  if (need > (size_t)GPTMI_STATIC_SCRATCH_BYTES) {
+    set_error("linear_static: these sizes need %zu bytes of packed operands, the built-in "
+              "scratch holds %zu; use gptmi_linear with a workspace, or pack the weight once "
+              "(GPTMI_W_PACKED)",
+              need, (size_t)GPTMI_STATIC_SCRATCH_BYTES);
+    return GPTMI_ERR_WORKSPACE;
+  }
+  void* ws = nullptr;
+  if (need > 0) {
+    ws = static_scratch();
+    if (ws == nullptr) return GPTMI_ERR_LAUNCH;
+  }
+  return linear_impl(x, W, bias, residual, out, M, N, K, gelu, p, seed, wlayout, ws,
+                     (size_t)GPTMI_STATIC_SCRATCH_BYTES, dtype, (hipStream_t)stream);
 }
 
 int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, void* k,

@@ -29,7 +29,10 @@
 extern "C" {
 #endif
 
-#define GPTMI_VERSION 100 /* major*10000 + minor*100 + patch */
+#define GPTMI_VERSION 101 /* major*10000 + minor*100 + patch */
+
+/* Size of the scratch array built into the library for gptmi_linear_static (8 MiB). */
+#define GPTMI_STATIC_SCRATCH_BYTES (8u << 20)
 
 typedef enum gptmi_dtype {
   GPTMI_F32 = 0, /* IEEE binary32 storage */
@@ -154,6 +157,28 @@ int gptmi_linear(const void* x, const void* W, const void* bias,
                  const void* residual, void* out, int64_t M, int64_t N, int64_t K,
                  int gelu, float p, uint64_t seed, int wlayout, void* workspace,
                  size_t workspace_bytes, int dtype, void* stream);
+
+/*
+ * gptmi_linear without the workspace arguments, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments, arithmetic, kernels and results as gptmi_linear;
+ * the packed operand images that gptmi_linear writes into the caller's workspace go into a
+ * GPTMI_STATIC_SCRATCH_BYTES array of device memory that is part of the library image (each GPU
+ * the library runs on holds it until the process ends).  The call allocates and frees nothing.
+ *   - Sizes whose gptmi_linear_workspace_bytes(M, N, K, dtype, wlayout) exceeds
+ *     gptmi_linear_static_capacity() are refused with GPTMI_ERR_WORKSPACE (fp16, K % 64 == 0,
+ *     W[K][N]: N*K*2 <= 8 MiB, e.g. every GEMM of GPT-2 124M; GPTMI_W_PACKED needs no scratch).
+ *   - Every call on a GPU shares that GPU's array and keeps nothing in it between calls (the
+ *     images are rewritten in full by each call).  Calls that overlap on one GPU -- two streams,
+ *     two host threads -- race on it; calls on one stream are ordered and safe.
+ *   - The first call on a device resolves the array's address there (hipGetSymbolAddress); make
+ *     that call outside a graph capture.
+ */
+size_t gptmi_linear_static_capacity(void);
+int gptmi_linear_static(const void* x, const void* W, const void* bias,
+                        const void* residual, void* out, int64_t M, int64_t N, int64_t K,
+                        int gelu, float p, uint64_t seed, int wlayout, int dtype,
+                        void* stream);
 
 /*
  * y = x @ W + bias with y's 3*heads*d columns split as [q | k | v] and each
