@@ -40,18 +40,38 @@ What pins each function (tests/test_oracle.py):
                against its closed form on the int32 edge values, the keep rate against p, and
                tests/golden/dropout.npz: outputs of the reference's fused_embeddings, fused_ffn
                and flash_attention_v1 with dropout_prob > 0 under Triton's CPU interpreter
+  fp32 chain   accumulation_dtype(np.float64) re-evaluates the same formulas with fp64 sums at
+               the same rounding points; tests/test_oracle.py measures how far that moves the
+               fp32-storage model output (the bound the GPU tests derive their tolerance from)
   model        an independently written fp64 torch GPT-2 (HF block order), and the
                transformers library's GPT2Model (random weights, built locally from a
                config) through the package's key conversion (test.py:120-133)
 No function of this file is left unpinned.
 """
+import contextlib
 import math
 
 import numpy as np
 
-F32 = np.float32
+F32 = np.float32  # the arithmetic type between rounding points; see accumulation_dtype
 F16 = np.float16
 BLOCK_L = 64  # K/V tile of the reference's attention kernel (kernels.py:509)
+
+
+@contextlib.contextmanager
+def accumulation_dtype(dtype):
+    """Inside the block every function of this file does its sums, products, exponentials and
+    normalisations in `dtype` (np.float64) instead of fp32, while every rounding point of the
+    reference stays where it is: operands still go through fp16, results are still stored in
+    the tensors' own dtype.  The distance between the two evaluations is the part of a result
+    that depends on nothing but the order and precision of fp32 accumulation -- the floor below
+    which two correct implementations of the reference's formulas cannot be told apart."""
+    global F32
+    saved, F32 = F32, dtype
+    try:
+        yield
+    finally:
+        F32 = saved
 
 
 def _as_f32(a):

@@ -60,21 +60,36 @@ def check(got, want, dtype, what=""):
                                  f"(max|diff| {diff.max():.3e}, max|ref| {scale:.3e})")
 
 
-def check_model_fp32(got, want, what=""):
+DRIFT_FACTOR = 3.0
+
+
+def fp32_chain_drift(params, ids, n_head, lm_head=False):
+    """The oracle's model outputs evaluated with fp64 sums at the same rounding points
+    (O.accumulation_dtype): the reference point for check_model_fp32."""
+    with O.accumulation_dtype(np.float64):
+        return O.gpt2_forward(params, ids, n_head, lm_head=lm_head)
+
+
+def check_model_fp32(got, want, want64, what=""):
     """End-to-end outputs in fp32 storage.  Every GEMM and the attention round their fp32 inputs
     to fp16 (kernels.py:229,234,414,428,465), so a last-bit difference in an activation (fp32
     sums are ordered differently on the GPU and in numpy) now and then flips one fp16 rounding,
     a 2^-11 relative step that the following layers carry along.  Each operator fed the
-    oracle's own intermediates is exact to ~1e-6 (test_gpt2_layerwise_fp32); chained, the
-    difference to the oracle settles around 1e-4 of max|b|.  Bounds: median <= 5e-4 * max|b|,
-    nothing beyond 5e-3 * max|b|."""
+    oracle's own intermediates is exact to ~1e-6 (test_gpt2_layerwise_fp32); chained, two
+    evaluations that differ in nothing but the precision of their sums -- the oracle with fp32
+    and with fp64 accumulation, `want` and `want64` -- end up a few 1e-4 of max|b| apart
+    (tests/test_oracle.py::test_fp32_chain_drift_is_accumulation_noise).  The GPU result may be
+    DRIFT_FACTOR times as far from `want` as `want64` is, in the maximum and in the median."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
+    want64 = np.asarray(want64, dtype=np.float64)
     assert got.shape == want.shape and np.all(np.isfinite(got)), what
-    scale = np.abs(want).max()
-    diff = np.abs(got - want)
-    assert diff.max() <= 5e-3 * scale, f"{what}: max|diff| {diff.max():.3e} (max|ref| {scale:.3e})"
-    assert np.median(diff) <= 5e-4 * scale, f"{what}: median |diff| {np.median(diff):.3e}"
+    diff, floor = np.abs(got - want), np.abs(want64 - want)
+    print(f"{what}: |gpu - oracle| max {diff.max():.3e} median {np.median(diff):.3e}; oracle fp64 vs "
+          f"fp32 sums: max {floor.max():.3e} median {np.median(floor):.3e}; max|ref| "
+          f"{np.abs(want).max():.3e}", flush=True)
+    assert diff.max() <= DRIFT_FACTOR * floor.max(), f"{what}: max|diff| {diff.max():.3e}"
+    assert np.median(diff) <= DRIFT_FACTOR * np.median(floor), f"{what}: median {np.median(diff):.3e}"
 
 
 def check_attention(got, want, v, dtype, what=""):
@@ -470,8 +485,9 @@ def test_gpt2_small_forward(gpu_device, dtype):
     hidden, logits = model(dev(ids, gpu_device), return_logits=True)
     want_h, want_l = O.gpt2_forward(params, ids, cfg["n_head"], lm_head=True)
     if dtype == torch.float32:
-        check_model_fp32(host(hidden), want_h, "hidden")
-        check_model_fp32(host(logits), want_l, "logits")
+        h64, l64 = fp32_chain_drift(params, ids, cfg["n_head"], lm_head=True)
+        check_model_fp32(host(hidden), want_h, h64, "hidden")
+        check_model_fp32(host(logits), want_l, l64, "logits")
     else:
         assert np.abs(host(hidden).astype(np.float64) - want_h).max() <= 2e-2
         assert np.abs(host(logits).astype(np.float64) - want_l).max() <= 2e-2
@@ -491,8 +507,9 @@ def test_gpt2_124m_config0(gpu_device, dtype):
     assert hidden.shape == (2, 64, 768) and logits.shape == (2, 64, 50257)
     want_h, want_l = O.gpt2_forward(params, ids, cfg["n_head"], lm_head=True)
     if dtype == torch.float32:
-        check_model_fp32(host(hidden), want_h, "hidden")
-        check_model_fp32(host(logits), want_l, "logits")
+        h64, l64 = fp32_chain_drift(params, ids, cfg["n_head"], lm_head=True)
+        check_model_fp32(host(hidden), want_h, h64, "hidden")
+        check_model_fp32(host(logits), want_l, l64, "logits")
     else:
         assert np.abs(host(hidden).astype(np.float64) - want_h).max() <= 2e-2
         assert np.abs(host(logits).astype(np.float64) - want_l).max() <= 2e-2
@@ -789,7 +806,9 @@ def test_gpt2_train_mode_forward(gpu_device, dtype):
     eval_want = O.gpt2_forward(params, ids, cfg["n_head"])
     assert np.abs(want.astype(np.float64) - eval_want).max() > 0.1  # the masks matter
     if dtype == torch.float32:
-        check_model_fp32(host(hidden), want, "hidden (train mode)")
+        with O.accumulation_dtype(np.float64):
+            want64 = O.gpt2_forward(params, ids, cfg["n_head"], dropout_prob=0.1)
+        check_model_fp32(host(hidden), want, want64, "hidden (train mode)")
     else:
         assert np.abs(host(hidden).astype(np.float64) - want).max() <= 2e-2
 
