@@ -59,8 +59,19 @@ def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
     return L * (gemm + attn) + (2 * tokens * h * arch["vocab_size"] if lm_head else 0)
 
 
-def cpu_baseline(sample_batch=16, reps=2):
-    import numpy as np
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
+def cpu_baseline(sample_batch=64, reps=3):
+    """PyTorch fp32 eager forward of the same 124M model on the host cores: 1 warm-up + `reps`
+    timed forwards of `sample_batch` x 300 tokens (about 15 s of CPU work on 16 cores)."""
     import torch
 
     from oracle import gpt2_oracle as O
@@ -74,15 +85,21 @@ def cpu_baseline(sample_batch=16, reps=2):
         seed=1337).items()}
     ids = torch.from_numpy(O.synthetic_ids(sample_batch, SEQLEN, ARCH["vocab_size"], seed=1337))
     gpt2_forward_fp32(params, ids, ARCH["n_head"])  # warm-up
-    t0 = time.perf_counter()
+    times = []
     for _ in range(reps):
+        t0 = time.perf_counter()
         gpt2_forward_fp32(params, ids, ARCH["n_head"])
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": round(sample_batch * SEQLEN / dt, 1), "unit": "tokens/s", "cores": threads,
-            "kind": "port",
-            "sample": f"PyTorch fp32 eager forward of the same 124M model on the host CPU, batch "
-                      f"{sample_batch} x seqlen {SEQLEN} ({sample_batch * SEQLEN} tokens), "
-                      f"mean of {reps} after 1 warm-up, {dt * 1e3:.0f} ms per forward"}
+        times.append(time.perf_counter() - t0)
+    mean, best = sum(times) / reps, min(times)
+    tokens = sample_batch * SEQLEN
+    return {"value": round(tokens / mean, 1), "unit": "tokens/s", "cores": threads,
+            "kind": "port", "cpu_model": cpu_model_name(), "logical_cores": cores,
+            "cpu_ms_mean": round(mean * 1e3, 1), "cpu_ms_min": round(best * 1e3, 1),
+            "cpu_tokens_per_s_best": round(tokens / best, 1),
+            "sample": f"PyTorch fp32 eager forward of the same 124M model on the host CPU "
+                      f"({threads} torch threads), batch {sample_batch} x seqlen {SEQLEN} "
+                      f"({tokens} tokens; the full 512 x 300 step would take ~{mean * 512 / sample_batch:.0f} s), "
+                      f"1 warm-up + {reps} timed forwards: mean {mean * 1e3:.0f} ms, min {best * 1e3:.0f} ms"}
 
 
 def copy_calibration(dev, rows=262144, cols=2048, reps=3):

@@ -35,6 +35,10 @@ static bool dropout_ok(float p) { return p >= 0.0f && p < 1.0f; }  // false for 
 
 static inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// Widest output row the GEMM epilogues address: their per-lane offsets cover up to 8 rows of N
+// elements of 4 bytes in an unsigned 32-bit register (8 * 2^26 * 4 = 2^31).
+constexpr int kMaxN = 1 << 26;
+
 // Workspace plan of one GEMM: where the packed weight and (if needed) the
 // packed activations live.
 struct LinearPlan {
@@ -163,8 +167,9 @@ static int check_linear_args(const void* x, const void* W, const void* out, int6
     set_error("linear: invalid argument");
     return GPTMI_ERR_INVALID;
   }
-  if (N > (1 << 30) || K > (1 << 30)) {
-    set_error("linear: N or K too large");
+  // the epilogues form per-lane byte offsets of up to 8 rows (8 * N * 4 bytes in fp32) in 32 bits
+  if (N > kMaxN || K > (1 << 30)) {
+    set_error("linear: N=%lld beyond %d or K=%lld beyond 2^30", (long long)N, kMaxN, (long long)K);
     return GPTMI_ERR_UNSUPPORTED;
   }
   if (!dropout_ok(p)) {
@@ -205,7 +210,7 @@ int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
     set_error("embed: dropout probability %g outside [0, 1)", (double)p);
     return GPTMI_ERR_INVALID;
   }
-  launch_embed(ids, wte, wpe, out, B * L, L, (int)H, Dropout{p, seed}, dtype == GPTMI_F16,
+  launch_embed(ids, wte, wpe, out, B * L, L, V, (int)H, Dropout{p, seed}, dtype == GPTMI_F16,
                (hipStream_t)stream);
   return check_launch("embed");
 }
@@ -315,8 +320,9 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, vo
     return GPTMI_ERR_UNSUPPORTED;
   }
   const int64_t M = B * L, N = 3 * heads * d;
-  if (N > (1 << 30) || K > (1 << 30)) {
-    set_error("linear_qkv: N or K too large");
+  if (N > kMaxN || K > (1 << 30)) {
+    set_error("linear_qkv: N=%lld beyond %d or K=%lld beyond 2^30", (long long)N, kMaxN,
+              (long long)K);
     return GPTMI_ERR_UNSUPPORTED;
   }
   hipStream_t st = (hipStream_t)stream;

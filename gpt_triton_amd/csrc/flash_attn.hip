@@ -68,11 +68,8 @@ __device__ __forceinline__ h8 zero_h8() {
 // D = head size.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
 // position c ^ (r&7)) and V^T tile [D][64] (8-byte unit u of row d at position
 // u ^ ((d>>1)&15)).
-#ifndef GPTMI_TILED_WAVES
-#define GPTMI_TILED_WAVES 2
-#endif
 template <int D, typename T, bool BLND, bool DROP>
-__global__ __launch_bounds__(256, (D == 64 && !DROP) ? GPTMI_TILED_WAVES : 1) void flash_attn_kernel(
+__global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     T* __restrict__ O, int heads, int L, float scale, DropoutArgs drop) {
   constexpr int CH = D / 8;             // 16-byte chunks per row
@@ -357,7 +354,6 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? GPTMI_TILED_WAVES : 1) vo
 // c/2 + 1 key tiles (causal), and the chunks are dealt to the wavefronts in snake
 // order from the most expensive one, which balances the triangle over the SIMDs
 // (L = 300: 8, 8, 7, 7 tiles).  The arithmetic per tile is that of the tiled kernel.
-// GPTMI_ATTN_NO_STAGE / GPTMI_ATTN_NO_COMPUTE are ablation switches of tuning builds.
 // ---------------------------------------------------------------------------
 template <int D, typename T, bool BLND, int NW>
 __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
@@ -390,11 +386,7 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
 #pragma unroll
   for (int i = 0; i < KI; ++i) {
     const int s = i * NT + tid;
-#ifdef GPTMI_ATTN_NO_STAGE
-    kr[i] = zero_h8();
-#else
     if (s < kchunks) kr[i] = Ld8<T>::load(Kp + (int64_t)(s / CH) * D + (s % CH) * 8);
-#endif
   }
 #pragma unroll
   for (int i = 0; i < VI; ++i) {
@@ -404,11 +396,7 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
     for (int kk = 0; kk < 4; ++kk) {
       int key = kg * 4 + kk;
       key = key < L ? key : L - 1;
-#ifdef GPTMI_ATTN_NO_STAGE
-      vr[i][kk] = zero_h8();
-#else
       if (u < units) vr[i][kk] = Ld8<T>::load(Vp + (int64_t)key * D + c * 8);
-#endif
     }
   }
 #pragma unroll
@@ -456,11 +444,7 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
       float mrun = -INFINITY, den = 0.f;
       int last_q = qw0 + 31;
       if (last_q > L - 1) last_q = L - 1;
-#ifdef GPTMI_ATTN_NO_COMPUTE
-      const int nt = L > (1 << 30) ? 1 : 0;
-#else
       const int nt = last_q / BKEY + 1;
-#endif
       for (int t = 0; t < nt; ++t) {
         const int k0 = t * BKEY;
         // ---- S^T = K . Q^T -----------------------------------------------------
@@ -593,10 +577,7 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
   }
 }
 
-#ifndef GPTMI_RESIDENT_WAVES
-#define GPTMI_RESIDENT_WAVES 8
-#endif
-constexpr int RESIDENT_WAVES = GPTMI_RESIDENT_WAVES;
+constexpr int RESIDENT_WAVES = 8;
 
 // LDS bytes of the resident variant, or 0 if this (L, D) does not fit two workgroups per CU.
 inline size_t resident_lds_bytes(int L, int D) {

@@ -61,9 +61,6 @@ struct EpiDev {
   int vec8_ok; // fp16 output: N, head size and the output pointers also allow 16-byte stores
   int m_off;   // head-major scatter: row 0 of this launch is row m_off of the [B*L] token rows
   DropoutArgs drop;  // p > 0: dropout between GELU and residual (predicated epilogue only)
-#ifdef GPTMI_TUNING
-  unsigned long long* trace;  // tuning builds only: per-workgroup phase time stamps
-#endif
 };
 
 // Direct global->LDS load of 16 bytes per lane: lane l's bytes land at LDS
@@ -83,7 +80,9 @@ __device__ __forceinline__ void lds_dma16(const void* gsrc, unsigned lds_off) {
 // byte offset: one VGPR per load instead of an address pair, and the k-step is a scalar add.
 __device__ __forceinline__ void lds_dma16_base(const void* base, unsigned lane_off,
                                                unsigned lds_off) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  // s_mov + s_nop 3 = 5 wait states between a VALU write of `base` (v_readfirstlane, should
+  // the compiler ever have to move it out of a vector register) and the load that reads it
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_off), "v"(lane_off), "s"(base)
                : "memory", "m0");
@@ -269,11 +268,6 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
           P4 o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = (T)z[e];
-#ifdef GPTMI_FAKE_STORE
-          *reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m & 255, n, N)) = o;
-#elif defined(GPTMI_PLAIN_STORE)
-          *reinterpret_cast<P4*>(out_ptr<T, QKV>(ep, m, n, N)) = o;
-#else
           // streaming store: the output is not read again by this kernel and
           // must not push the operand panels out of L2
           T* dst;
@@ -292,7 +286,6 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
             dst = out_ptr<T, QKV>(ep, m, n, N);
           }
           __builtin_nontemporal_store(o, reinterpret_cast<P4*>(dst));
-#endif
         } else {
           if (m >= M || n >= N) continue;
           T* op = out_ptr<T, QKV>(ep, m, n, N);
@@ -554,10 +547,6 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   // (the base addresses of the epilogue's stores) is scalar arithmetic in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % WM, wn = wave / WM;
-#ifdef GPTMI_TUNING
-  const unsigned long long t_start = __builtin_amdgcn_s_memtime();
-  const unsigned long long r_start = __builtin_amdgcn_s_memrealtime();
-#endif
   // Tile order: the column tiles are cut into groups of group_w; inside a group the column
   // runs fastest, then the row block, and the groups follow each other.  Workgroups that run
   // at the same time then share few weight panels, which stay in the XCD's L2.
@@ -661,11 +650,6 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   };
 
   const int KT = Kp / BKS;
-#ifdef GPTMI_NO_LOADS
-  constexpr bool loads = false;
-#else
-  constexpr bool loads = true;
-#endif
   // Residual through LDS.  Half h = rows 64 h .. 64 h + 63 of the wavefront's sub-tile goes
   // to this wavefront's own 8 KB of operand stage `stg`: 8 direct loads of 8 rows, lane l of
   // load q fetching 16-byte unit (l % 8) ^ key of row r = 8 q + l / 8, key = (r >> 1) & 7 =
@@ -693,19 +677,14 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   // landed, own LDS reads retired, barrier), its first fragments are requested, and the stage of
   // tile kt, which nobody reads any more, is refilled with tile kt+NST while that last slice is
   // multiplied.  No MFMA ever waits for a barrier plus an LDS round trip.
-  if (loads) {
 #pragma unroll
-    for (int s = 0; s < NST; ++s)
-      if (s < KT) issue(s);
-    // tile 0 must have landed; up to NST-1 younger tiles stay in flight
-    if (KT >= NST) wait_vmcnt<(NST - 1) * LPT>();
-    else wait_vmcnt<0>();
-  }
+  for (int s = 0; s < NST; ++s)
+    if (s < KT) issue(s);
+  // tile 0 must have landed; up to NST-1 younger tiles stay in flight
+  if (KT >= NST) wait_vmcnt<(NST - 1) * LPT>();
+  else wait_vmcnt<0>();
   asm volatile("s_barrier" ::: "memory");
   read_frags(0, 0, 0);
-#ifdef GPTMI_TUNING
-  const unsigned long long t_pro = __builtin_amdgcn_s_memtime();
-#endif
 
   for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
@@ -715,25 +694,15 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       if (!last) {
         read_frags(kt, ks + 1, cur ^ 1);
       } else if (kt + 1 < KT) {
-        if (loads) {
-          // tile kt+1 complete; tiles kt+2 .. kt+NST-1 may still be in flight
-          if (kt + NST - 1 < KT) wait_vmcnt<(NST - 2) * LPT>();
-          else wait_vmcnt<0>();
-        }
+        // tile kt+1 complete; tiles kt+2 .. kt+NST-1 may still be in flight
+        if (kt + NST - 1 < KT) wait_vmcnt<(NST - 2) * LPT>();
+        else wait_vmcnt<0>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         read_frags(kt + 1, 0, cur ^ 1);
       }
       __builtin_amdgcn_sched_barrier(0);
-#ifndef GPTMI_NO_MFMA
-      if (last) mma_and_issue(cur, kt + NST, kt + NST < KT && loads);
+      if (last) mma_and_issue(cur, kt + NST, kt + NST < KT);
       else mma(cur);
-#else
-#pragma unroll
-      for (int j = 0; j < MB; ++j) acc[0][j][0] += (float)af[cur][j][0] + (float)af[cur][j][7];
-#pragma unroll
-      for (int i = 0; i < NB; ++i) acc[i][0][1] += (float)bf[cur][i][0] + (float)bf[cur][i][7];
-      if (last && kt + NST < KT && loads) issue(kt + NST);
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (RESLDS) {
@@ -746,21 +715,6 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   }
 
   // ---- epilogue -----------------------------------------------------------
-#ifdef GPTMI_TUNING
-  const unsigned long long t_loop = __builtin_amdgcn_s_memtime();
-#endif
-#ifdef GPTMI_NO_EPILOGUE
-  {
-    float keep = 0.f;  // consumes every accumulator so that no MFMA is dead code
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int j = 0; j < MB; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) keep += acc[i][j][r];
-    if (keep == 123.456f) ((T*)ep.out)[tid] = (T)keep;
-  }
-#else
   block_barrier();  // every wavefront is done reading the operand stages
   const bool fast = ep.vec_ok && n0 + BN <= N && m0 + BM <= M;
   bool stored = false;
@@ -807,25 +761,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     store_wave_tile<MB, NB, T, QKV>(acc, ep, (int64_t)m0 + wm * TM + moff, n0 + wn * TN, M + moff,
                                     N, fast, smem + wave * EP_SLAB, lane);
   }
-#endif
-#ifdef GPTMI_TUNING
-  if (ep.trace && tid == 0) {
-    // shader-clock stamps of the phases, and the constant 100 MHz clock around the whole
-    // workgroup (the ratio of the two spans is the shader clock the workgroup ran at)
-    unsigned long long* t = ep.trace + (size_t)blockIdx.x * 6;
-    t[0] = t_start;
-    t[1] = t_pro;
-    t[2] = t_loop;
-    t[3] = __builtin_amdgcn_s_memtime();
-    t[4] = r_start;
-    t[5] = __builtin_amdgcn_s_memrealtime();
-  }
-#endif
 }
-
-#ifdef GPTMI_TUNING
-int g_group_w = 0;
-#endif
 
 // Width, in column tiles, of the groups the tile order walks through.  The weight panels of
 // one group (group_w * BN rows of Kp halves) should stay in a 4 MB L2 beside the activation
@@ -857,10 +793,7 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
     attr_done = true;
   }
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (N + BN - 1) / BN;
-  int group_w = column_group(tiles_n, BN, Kp);
-#ifdef GPTMI_TUNING
-  if (g_group_w > 0) group_w = g_group_w < tiles_n ? g_group_w : tiles_n;
-#endif
+  const int group_w = column_group(tiles_n, BN, Kp);
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(WM * WN * 64), smem, st,
                      (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n,
                      group_w, ep);
@@ -1191,10 +1124,7 @@ int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const
   if (num_cus < 0) return num_cus;
   const int tiles_m = (int)((M + 255) / 256), tiles_n = (N + 255) / 256;
   const int num_tiles = tiles_m * tiles_n;
-  int group_w = column_group(tiles_n, 256, Kp);
-#ifdef GPTMI_TUNING
-  if (g_group_w > 0) group_w = g_group_w < tiles_n ? g_group_w : tiles_n;
-#endif
+  const int group_w = column_group(tiles_n, 256, Kp);
   const int grid = num_tiles < num_cus ? num_tiles : num_cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, st, (const _Float16*)A,
                      (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n, group_w, ep);
@@ -1247,7 +1177,6 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
 
 }  // namespace
 
-#ifndef GPTMI_TUNING
 int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const GemmEpilogue& e,
                 hipStream_t st) {
   if (M >= (1ll << 31) - 512) {
@@ -1285,6 +1214,5 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const G
   return e.qkv ? launch_shape<float, true>(A, Bt, M, N, Kp, ep, st)
                : launch_shape<float, false>(A, Bt, M, N, Kp, ep, st);
 }
-#endif
 
 }  // namespace gptmi

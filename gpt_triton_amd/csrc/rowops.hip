@@ -19,27 +19,30 @@ template <> struct Vec<float> {
 // ---------------------------------------------------------------------------
 // Embedding gather: out[row,:] = wte[ids[row],:] + wpe[row % L,:]
 // (reference: fused_embeddings_kernel, kernels.py:37-72).  The add is done in
-// fp32 and rounded once, which equals one add in the storage dtype.
+// fp32 and rounded once, which equals one add in the storage dtype.  A token id
+// outside [0, V) reads nothing: its wte row counts as zeros (the reference reads
+// out of bounds there).
 // ---------------------------------------------------------------------------
 template <typename T, int LPR>
 __global__ __launch_bounds__(256) void embed_vec_kernel(
     const int64_t* __restrict__ ids, const T* __restrict__ wte,
-    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H) {
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int64_t V_, int H) {
   typedef typename Vec<T>::type V;
   constexpr int VN = Vec<T>::N;
   const int lane = threadIdx.x & (LPR - 1);  // LPR lanes per token, as in the LayerNorm kernel
   const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
   if (row >= rows) return;
   const int64_t tok = ids[row];
+  const bool known = (uint64_t)tok < (uint64_t)V_;
   const int64_t pos = row % L;
-  const V* a = reinterpret_cast<const V*>(wte + tok * H);
+  const V* a = reinterpret_cast<const V*>(wte + (known ? tok : 0) * H);
   const V* b = reinterpret_cast<const V*>(wpe + pos * H);
   V* o = reinterpret_cast<V*>(out + row * H);
   const int nchunks = H / VN;
   for (int c = lane; c < nchunks; c += LPR) {
     V va = a[c], vb = b[c], vo;
 #pragma unroll
-    for (int j = 0; j < VN; ++j) vo[j] = (T)((float)va[j] + (float)vb[j]);
+    for (int j = 0; j < VN; ++j) vo[j] = (T)((known ? (float)va[j] : 0.f) + (float)vb[j]);
     __builtin_nontemporal_store(vo, o + c);
   }
 }
@@ -47,14 +50,15 @@ __global__ __launch_bounds__(256) void embed_vec_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void embed_scalar_kernel(
     const int64_t* __restrict__ ids, const T* __restrict__ wte,
-    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H) {
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int64_t V_, int H) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int64_t tok = ids[row];
+  const bool known = (uint64_t)tok < (uint64_t)V_;
   const int64_t pos = row % L;
   for (int c = lane; c < H; c += 64)
-    out[row * H + c] = (T)((float)wte[tok * H + c] + (float)wpe[pos * H + c]);
+    out[row * H + c] = (T)((known ? (float)wte[tok * H + c] : 0.f) + (float)wpe[pos * H + c]);
 }
 
 // Embedding with dropout (kernels.py:65-70): the sum is rounded to the storage dtype first,
@@ -63,15 +67,16 @@ __global__ __launch_bounds__(256) void embed_scalar_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void embed_dropout_kernel(
     const int64_t* __restrict__ ids, const T* __restrict__ wte,
-    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int H,
+    const T* __restrict__ wpe, T* __restrict__ out, int64_t rows, int64_t L, int64_t V_, int H,
     DropoutArgs drop) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int64_t tok = ids[row];
+  const bool known = (uint64_t)tok < (uint64_t)V_;
   const int64_t pos = row % L;
   for (int c = lane; c < H; c += 64) {
-    const T sum = (T)((float)wte[tok * H + c] + (float)wpe[pos * H + c]);
+    const T sum = (T)((known ? (float)wte[tok * H + c] : 0.f) + (float)wpe[pos * H + c]);
     unsigned off[1] = {(unsigned)c};
     float z[1] = {(float)sum};
     dropout_apply<1>(drop, off, z);
@@ -310,7 +315,7 @@ static inline int lanes_per_row(int nchunks) {
 
 template <typename T>
 static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
-                          void* out, int64_t rows, int64_t L, int H, Dropout drop,
+                          void* out, int64_t rows, int64_t L, int64_t V, int H, Dropout drop,
                           hipStream_t st) {
   const unsigned grid = (unsigned)((rows + 3) / 4);
   // The reference runs the dropout even at p = 0 (kernels.py:70), where it is the identity
@@ -319,7 +324,7 @@ static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
   if (drop.p != 0.0f || drop.seed != 1337 || H > (1 << 20)) {
     const DropoutArgs d = {drop.p, (unsigned)drop.seed, (unsigned)(drop.seed >> 32)};
     hipLaunchKernelGGL(embed_dropout_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
-                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H, d);
+                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, V, H, d);
     return 0;
   }
   const bool aligned = (H % Vec<T>::N) == 0 && ((uintptr_t)wte % 16) == 0 &&
@@ -327,20 +332,21 @@ static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
   if (aligned)
     if (lanes_per_row(H / Vec<T>::N) == 32)
       hipLaunchKernelGGL((embed_vec_kernel<T, 32>), dim3((unsigned)((rows + 7) / 8)), dim3(256), 0,
-                         st, ids, (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+                         st, ids, (const T*)wte, (const T*)wpe, (T*)out, rows, L, V, H);
     else
       hipLaunchKernelGGL((embed_vec_kernel<T, 64>), dim3(grid), dim3(256), 0, st, ids,
-                         (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+                         (const T*)wte, (const T*)wpe, (T*)out, rows, L, V, H);
   else
     hipLaunchKernelGGL(embed_scalar_kernel<T>, dim3(grid), dim3(256), 0, st, ids,
-                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, H);
+                       (const T*)wte, (const T*)wpe, (T*)out, rows, L, V, H);
   return 0;
 }
 
 int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
-                 int64_t rows, int64_t L, int H, Dropout drop, bool f16, hipStream_t st) {
-  return f16 ? launch_embed_t<_Float16>(ids, wte, wpe, out, rows, L, H, drop, st)
-             : launch_embed_t<float>(ids, wte, wpe, out, rows, L, H, drop, st);
+                 int64_t rows, int64_t L, int64_t V, int H, Dropout drop, bool f16,
+                 hipStream_t st) {
+  return f16 ? launch_embed_t<_Float16>(ids, wte, wpe, out, rows, L, V, H, drop, st)
+             : launch_embed_t<float>(ids, wte, wpe, out, rows, L, V, H, drop, st);
 }
 
 template <typename T, int CH>

@@ -73,8 +73,8 @@ const char* gptmi_last_error(void);
  * Replaces fused_embeddings(x, wte, wpe, dropout_prob) -> kernels.py:75-101 and
  * fused_embeddings_kernel -> kernels.py:37-72.
  *   ids  int64 [B*L]          wte [V][H]     wpe [P][H]     out [B*L][H]
- * Requires L <= P.  Token ids are NOT range checked on the device (neither does
- * the reference); the host wrapper may check them.
+ * Requires L <= P.  A token id outside [0, V) reads no memory: its wte row counts as zeros, so
+ * the output row is wpe[l,:] (the reference does not check and reads out of bounds).
  * Dropout (0 <= p < 1, dropout() -> kernels.py:31-34): the sum, rounded to the storage
  * dtype, is kept where rand(seed, column) > p and divided by (1 - p), else zeroed; rand is
  * Triton's tl.rand, i.e. Philox-4x32-10 with counter (column, 0, 0, 0), the 64-bit seed as
@@ -146,7 +146,8 @@ int gptmi_pack_weight(const void* W, void* packed, int64_t N, int64_t K, int wla
  *                               element is read before it is written)
  * workspace: at least gptmi_linear_workspace_bytes(...) bytes, 256-byte aligned
  * (may be NULL when that is 0).
- * Any M, N, K >= 1 and any pointer alignment the element type allows are accepted; the fast
+ * Any M >= 1 (below 2^31 - 512), 1 <= N <= 2^26, 1 <= K <= 2^30 (GPTMI_ERR_UNSUPPORTED beyond)
+ * and any pointer alignment the element type allows are accepted; the fast
  * epilogues need N a multiple of 8 (fp16) or 4 (fp32) and 16-byte aligned bias, residual and
  * out, everything else takes element-wise code with the same results.
  * Dropout (0 < p < 1; 0 = none) sits between the GELU and the residual

@@ -134,6 +134,26 @@ def test_fused_embeddings_gpt2_shape(K, gpu_device, dtype):
     assert np.array_equal(host(z), O.fused_embeddings(ids, wte, wpe))
 
 
+def test_fused_embeddings_out_of_range_ids_read_nothing(K, gpu_device):
+    """Token ids outside [0, V) -- negative, V itself, far beyond -- count as a zero wte row
+    (the output row is the position embedding); the rows around them are unaffected."""
+    r = np.random.default_rng(9)
+    V, H, P, B, L = 50, 768, 16, 2, 8
+    ids = r.integers(0, V, size=(B, L))
+    bad = [(0, 1, -1), (0, 5, V), (1, 0, 1 << 40), (1, 7, -(1 << 62))]
+    for dtype in (torch.float16, torch.float32):
+        wte = r.standard_normal((V, H)).astype(NP[dtype])
+        wpe = r.standard_normal((P, H)).astype(NP[dtype])
+        ids_bad = ids.copy()
+        for b, l, v in bad:
+            ids_bad[b, l] = v
+        want = O.fused_embeddings(ids, wte, wpe)
+        for b, l, _ in bad:
+            want[b, l] = wpe[l]
+        z = K.fused_embeddings(dev(ids_bad, gpu_device), dev(wte, gpu_device), dev(wpe, gpu_device))
+        assert np.array_equal(host(z), want)
+
+
 # ----------------------------------------------------------------------------- layer norm
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("M", [249, 32])

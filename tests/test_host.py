@@ -58,6 +58,15 @@ def test_invalid_arguments_are_rejected_before_any_launch(lib):
                                 None) == -1                                             # p < 0
     assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 9, 64, 0.125, 0.0, 0, 0, 1,
                                 None) == -2                                             # Lq != Lk
+    # output rows wider than the epilogues' 32-bit lane offsets can address: refused, not wrapped
+    wide = (1 << 26) + 8
+    assert lib.gptmi_linear(fake, fake, None, None, fake, 4, wide, 64, 0, 0.0, 0, 2, None, 0, 1,
+                            None) == -2
+    assert b"N=" in lib.gptmi_last_error()
+    assert lib.gptmi_linear_static(fake, fake, None, None, fake, 4, wide, 64, 0, 0.0, 0, 2, 1,
+                                   None) == -2
+    assert lib.gptmi_linear_qkv(fake, fake, None, fake, fake, fake, 1, 4, 1 << 20, 64, 64, 2,
+                                None, 0, 1, None) == -2                    # N = 3 * 2^26
     assert lib.gptmi_linear(fake, fake, None, None, fake, 4, 4, 4, 0, 0.0, 0, 0, None, 0, 1,
                             None) == -3                                                 # workspace
 
