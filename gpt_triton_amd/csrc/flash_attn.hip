@@ -22,6 +22,8 @@
 // LDS (4 keys x 8 d per thread, register transpose, 8-byte stores).
 // Wavefronts 0-1 stage the K tile, wavefronts 2-3 stage V^T; the next tile's
 // global loads are in flight while the current one is consumed.
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
 
@@ -577,6 +579,363 @@ __global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Streaming variant of the resident kernel: fp16 storage, head size 64, K and V of one (batch,
+// head) no larger than 320 rows (two of them fill the CU's 160 KB of LDS).
+//
+// One persistent workgroup of 8 wavefronts per CU walks (batch, head) pairs bh = blockIdx.x,
+// blockIdx.x + gridDim.x, ...  K and V of pair i+1 are brought into the second half of LDS by
+// direct global->LDS loads (16 bytes per lane, no staging registers, no LDS store instructions)
+// while pair i is multiplied, so HBM is kept busy through the arithmetic; the one barrier per
+// pair publishes the buffer that has landed and frees the other.  The queries of pair i+1 are
+// requested early in the iteration as well (see the pipeline at the end of the kernel).
+//
+// LDS, per buffer: K [Lp][64] then V [Lp][64] halves, Lp = L rounded up to 64, rows of 128 bytes
+// in 16-byte units.  The loads write LDS in lane order, so the swizzle is applied on the source
+// side: unit u of K row r holds source unit u ^ ((r >> 1) & 7) (conflict-free ds_read_b128 of one
+// unit of 32 consecutive rows), unit u of V row r holds source unit u ^ (2 (r & 3)).  V stays
+// row-major: the first operand of O^T += V^T . P^T is read with the transposing LDS load
+// (ds_read_b64_tr_b16: within a block of 16 lanes, lane i receives element i % 4 of the 8 bytes
+// addressed by lanes i / 4, i / 4 + 4, + 8, + 12), lane s of a block pointing at V[key0 + s / 4]
+// [d0 + 4 (s % 4) ..]; the V swizzle spreads the four rows of such a block over all banks.
+// Rows L .. Lp-1 are filled with copies of row L-1: their keys are masked (P = 0 exactly) and
+// the values are finite.
+//
+// The causal diagonal is handled per 32 x 32 block instead of per 64-key tile.  The first query
+// of a 32-query chunk is a multiple of 32, so in the chunk's last key tile one 32-key block is
+// cut by the diagonal -- the same lanes and registers are masked in every chunk, by a compare
+// against a constant and a select per score -- and the other block is either
+// entirely visible (no mask) or entirely hidden (skipped: its weights are exactly 0 and add
+// exactly 0 to the sums, so leaving it out changes no bit of the result).
+//
+// Chunk c costs c + 1 such blocks; the host deals the chunks to the 8 wavefronts (at most two
+// each) so that the four SIMDs -- wavefronts w and w + 4 share one -- carry equal block counts.
+// ---------------------------------------------------------------------------
+struct StreamPlan {
+  signed char chunk[8][2];  // query chunks (of 32) of wavefront w, -1 = none
+};
+
+typedef short s4v __attribute__((__vector_size__(4 * sizeof(short))));
+
+// four keys x one d (transposed) from a row-major V tile; see the layout note above
+__device__ __forceinline__ h4 lds_read_tr16(const char* p) {
+  const s4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s4v*)(uintptr_t)p);
+  return __builtin_bit_cast(h4, r);
+}
+
+// 16 bytes per lane from (wavefront-uniform base) + lane_off straight into LDS at lds_off +
+// 16 * lane.  Assembly, so that the compiler's wait-count model never sees an LDS-writing memory
+// operation in flight (it would make every LDS read of the arithmetic wait for the prefetch);
+// completion is awaited by hand (vmcnt(0)) in front of the barrier that publishes the buffer.
+__device__ __forceinline__ void attn_dma16(const void* base, unsigned lane_off, unsigned lds_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_off), "v"(lane_off), "s"(base)
+               : "memory", "m0");
+}
+
+template <bool BLND>
+__global__ __launch_bounds__(512, 2) void flash_attn_stream_kernel(
+    const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+    const _Float16* __restrict__ V, _Float16* __restrict__ O, int heads, int L, int num_bh,
+    float scale, StreamPlan plan) {
+  constexpr int D = 64, KS = 4, DB = 2;
+  constexpr int MAX_DMA = 10;  // 16-byte loads per lane per pair: Lp / 32, Lp <= 320
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int Lp = (L + BKEY - 1) / BKEY * BKEY;
+  const int buf_bytes = Lp * 256;  // K then V, 128 bytes per row
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ql = lane & 31, g = lane >> 5;
+  const unsigned smem_base = (unsigned)(uintptr_t)smem;
+
+  // ---- what this wavefront loads: units [(wave * ndma + j) * 64 + lane] of the Lp * 16 units of
+  // K followed by V (ndma = Lp / 32 loads per wavefront and pair, the same for all wavefronts)
+  const int ndma = Lp >> 5;
+  const int k_loads = Lp >> 3;  // the first Lp / 8 of the workgroup's 8 * ndma loads fill K
+  // load `inst` covers rows 8 * inst' .. + 7 (inst' counted from the start of K or of V); lane l
+  // fills position l % 8 of row 8 * inst' + l / 8 with source unit (l % 8) ^ key(row):
+  // K key = (row >> 1) & 7 = (4 * (inst' & 1) + l / 16) & 7, V key = 2 * (row & 3) = 2 * ((l / 8) & 3)
+  const int lrow = lane >> 3;
+  const unsigned k_unit16 = (unsigned)(((lane & 7) ^ (lane >> 4)) << 4);
+  const unsigned v_unit16 = (unsigned)(((lane & 7) ^ (2 * (lrow & 3))) << 4);
+  auto issue_pair = [&](int bh, int buf) {
+    const char* kb_ = (const char*)(K + (int64_t)bh * L * D);
+    const char* vb_ = (const char*)(V + (int64_t)bh * L * D);
+    const unsigned dst = smem_base + (unsigned)(buf * buf_bytes) + (unsigned)(wave * ndma) * 1024u;
+#pragma unroll
+    for (int j = 0; j < MAX_DMA; ++j)
+      if (j < ndma) {
+        const int inst = wave * ndma + j;
+        const bool is_v = inst >= k_loads;
+        const int rel = inst - (is_v ? k_loads : 0);
+        int row = rel * 8 + lrow;
+        row = row < L ? row : L - 1;  // rows L .. Lp-1 repeat the last row
+        const unsigned unit16 = is_v ? v_unit16 : (k_unit16 ^ ((unsigned)(rel & 1) << 6));
+        attn_dma16(is_v ? vb_ : kb_, (unsigned)row * 128u + unit16, dst + j * 1024);
+      }
+  };
+
+  // ---- this wavefront's query chunks and their fragments: lane (ql, g) holds d = 16 ks + 8 g + 0..7
+  const int c0 = plan.chunk[wave][0], c1 = plan.chunk[wave][1];
+  auto load_q = [&](int bh, int c, h8 (&qf)[KS]) {
+    int q = c * 32 + ql;
+    q = q < L ? q : L - 1;  // rows past the end are computed and never stored
+    const _Float16* qp = Q + ((int64_t)bh * L + q) * D + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const h8*>(qp + ks * 16);
+  };
+
+  // ---- the block cut by the diagonal: register r of a 32 x 32 score block is key offset
+  // 8 (r / 4) + 4 g + r % 4, visible to query offset ql iff that is <= ql -- the same lanes and
+  // registers in every chunk
+  const int tri_q = ql - 4 * g;
+
+  // ---- LDS read offsets (bytes inside a buffer) of this lane
+  // K fragment of 32-key block at row k: row k + ql, unit (2 ks + g) ^ ((ql >> 1) & 7)
+  int k_off[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) k_off[ks] = ql * 128 + (((ks * 2 + g) ^ ((ql >> 1) & 7)) << 4);
+  // V^T fragment of d block i, keys key0 + 4 g + 0..3: lane s = lane % 16 of its block of 16 points
+  // at V[key0 + 4 g + s / 4][32 i + 16 (block % 2) + 4 (s % 4)]
+  const int sl = lane & 15, vrow = 4 * g + (sl >> 2);
+  int v_off[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int unit = 4 * i + 2 * ((lane >> 4) & 1) + ((sl & 3) >> 1);
+    v_off[i] = Lp * 128 + vrow * 128 + ((unit ^ (2 * (vrow & 3))) << 4) + (sl & 1) * 8;
+  }
+  const float cexp = scale * 1.4426950408889634f;
+
+  // K fragments of the 64-key tile at row k0: [kb][ks]
+  auto read_k = [&](const char* buf, int k0, h8 (&kf)[2][KS]) {
+    const char* kt = buf + k0 * 128;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kf[kb][ks] = *reinterpret_cast<const h8*>(kt + kb * 4096 + k_off[ks]);
+  };
+
+  // One 64-key tile of one chunk.  MODE 0: both 32-key blocks entirely visible; 1: block 0 cut
+  // by the diagonal, block 1 hidden (skipped); 2: block 0 visible, block 1 cut by the diagonal.
+  // The K fragments arrive in registers (read one step ahead); the V^T fragments and, if
+  // `more`, the next tile's K fragments are requested right behind the score products, so that
+  // the LDS round trips run under the softmax arithmetic and no product waits for one.  The
+  // scheduling fences keep the compiler from sinking the reads back down to their uses.
+  auto step = [&](auto mode_tag, const char* buf, int k0, bool more, h8 (&kf)[2][KS],
+                  const h8 (&qf)[KS], f16v (&oacc)[DB], float& mrun, float& den) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr int NKB = MODE == 1 ? 1 : 2;
+    f16v s[NKB];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[kb][ks], qf[ks], s[kb], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // this lane group's keys of a 16-key step: base + 4 g + 0..3 (lo) and base + 8 + 4 g + 0..3 (hi);
+    // block 0's fragments are requested here, block 1's when block 0's products start
+    h4 vlo[2][DB], vhi[2][DB];
+    auto read_v = [&](int kb) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const char* vt = buf + (k0 + kb * 32 + tt * 16) * 128;
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+          vlo[tt][i] = lds_read_tr16(vt + v_off[i]);
+          vhi[tt][i] = lds_read_tr16(vt + v_off[i] + 8 * 128);
+        }
+      }
+    };
+    read_v(0);
+    if (more) read_k(buf, k0 + BKEY, kf);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (MODE != 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s[NKB - 1][r] = 8 * (r >> 2) + (r & 3) <= tri_q ? s[NKB - 1][r] : -INFINITY;
+    }
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, s[kb][r]);
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+    const float mnew = bmax > mrun ? bmax : mrun;
+    const float mult = __builtin_amdgcn_exp2f((mrun - mnew) * cexp);
+    const float m2 = mnew * cexp;
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][r], cexp, -m2));
+        s[kb][r] = p;
+        psum += p;
+      }
+    mrun = mnew;
+    psum += __shfl_xor(psum, 32, kWave);
+    den = den * mult + psum;
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] *= mult;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      h8 vf[2][DB];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+          const h4 lo = vlo[tt][i], hi = vhi[tt][i];
+          vf[tt][i] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      if (kb + 1 < NKB) {  // the registers are free again: request the next block's fragments
+        __builtin_amdgcn_sched_barrier(0);
+        read_v(kb + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        h8 pf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pf[j] = (_Float16)s[kb][8 * tt + j];
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[tt][i], pf, oacc[i], 0, 0, 0);
+      }
+    }
+  };
+
+  auto run_chunk = [&](int bh, int c, const char* buf, const h8 (&qf)[KS]) {
+    const int qw0 = c * 32, q = qw0 + ql;
+    f16v oacc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float mrun = -INFINITY, den = 0.f;
+    const int nfull = qw0 >> 6;  // key tiles entirely below the diagonal
+    h8 kf[2][KS];
+    read_k(buf, 0, kf);
+    for (int t = 0; t < nfull; ++t)
+      step(std::integral_constant<int, 0>{}, buf, t * BKEY, true, kf, qf, oacc, mrun, den);
+    if ((qw0 & 32) == 0)
+      step(std::integral_constant<int, 1>{}, buf, nfull * BKEY, false, kf, qf, oacc, mrun, den);
+    else
+      step(std::integral_constant<int, 2>{}, buf, nfull * BKEY, false, kf, qf, oacc, mrun, den);
+    // Output.  A lane holds, per 8 consecutive d, the first (g = 0) or the second (g = 1) four of
+    // its query's row; the two lanes of a query trade halves through the 32-lane swap (the upper
+    // half of the first operand against the lower half of the second), after which each owns 8
+    // consecutive d of every other group: 4 stores of 16 bytes per lane instead of 8 of 8, and
+    // 32 contiguous bytes per row and instruction.
+    const float inv = __builtin_amdgcn_rcpf(den);
+    u4 out[DB][2];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        h4 x, y;  // d = 32 i + 16 pr + 4 g + 0..3 and the same + 8
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[j] = (_Float16)(oacc[i][8 * pr + j] * inv);
+          y[j] = (_Float16)(oacc[i][8 * pr + 4 + j] * inv);
+        }
+        const u2 xd = __builtin_bit_cast(u2, x), yd = __builtin_bit_cast(u2, y);
+        const auto r0 = __builtin_amdgcn_permlane32_swap(xd[0], yd[0], false, false);
+        const auto r1 = __builtin_amdgcn_permlane32_swap(xd[1], yd[1], false, false);
+        // g = 0: own x, then the partner's x (d + 4..7); g = 1: the partner's y, then own y
+        out[i][pr] = u4{r0[0], r1[0], r0[1], r1[1]};
+      }
+    if (q < L) {
+      int64_t row_off;
+      if (BLND) {
+        const int b = bh / heads, n = bh - b * heads;
+        row_off = (((int64_t)b * L + q) * heads + n) * D;
+      } else {
+        row_off = ((int64_t)bh * L + q) * D;
+      }
+#pragma unroll
+      for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr)
+          *reinterpret_cast<u4*>(O + row_off + i * 32 + 16 * pr + 8 * g) = out[i][pr];
+    }
+  };
+
+  // ---- the pipeline over this workgroup's pairs.  A wavefront's first chunk is its heavy one;
+  // the light one (if any) runs first, so that both sets of queries for the next pair are
+  // requested early in the iteration: the heavy chunk's into a second register set right behind
+  // the K / V loads, the light chunk's into its own registers when it is done with them.
+  h8 q_heavy[KS], q_heavy_next[KS], q_light[KS];
+  int bh = blockIdx.x;
+  if (bh >= num_bh) return;
+  issue_pair(bh, 0);
+  if (c0 >= 0) load_q(bh, c0, q_heavy_next);
+  if (c1 >= 0) load_q(bh, c1, q_light);
+  int buf = 0;
+  while (true) {
+    const int bh_next = bh + (int)gridDim.x;
+    const bool has_next = bh_next < num_bh;
+    // everything this wavefront requested has landed (the pair's K / V units and queries, and
+    // the previous pair's stores); behind the barrier that holds for every wavefront, and
+    // nobody reads the other buffer any more
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // The compiler cannot see the wait above.  Touching this pair's query registers here makes
+    // it place its own wait for them at this point, where it costs nothing; otherwise it would
+    // wait at their first use, inside the tile loop, with a count that knows nothing of the
+    // prefetch loads issued below, i.e. until those have landed too.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+v"(q_heavy_next[ks]));
+      asm volatile("" : "+v"(q_light[ks]));
+      q_heavy[ks] = q_heavy_next[ks];
+    }
+    if (has_next) {
+      issue_pair(bh_next, buf ^ 1);
+      if (c0 >= 0) load_q(bh_next, c0, q_heavy_next);
+    }
+    const char* b_ = smem + buf * buf_bytes;
+    if (c1 >= 0) {
+      run_chunk(bh, c1, b_, q_light);
+      if (has_next) load_q(bh_next, c1, q_light);
+    }
+    if (c0 >= 0) run_chunk(bh, c0, b_, q_heavy);
+    if (!has_next) break;
+    bh = bh_next;
+    buf ^= 1;
+  }
+}
+
+// Deals the query chunks of a sequence of L <= 320 rows to the 8 wavefronts: chunk c costs
+// c + 1 blocks; heaviest first, each to the SIMD (wavefronts w and w + 4) with the smallest
+// load so far that still has a free slot, inside the SIMD to the lighter wavefront.
+inline StreamPlan make_stream_plan(int L) {
+  StreamPlan p;
+  int wave_load[8] = {0, 0, 0, 0, 0, 0, 0, 0}, wave_n[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int w = 0; w < 8; ++w) p.chunk[w][0] = p.chunk[w][1] = -1;
+  for (int c = (L + 31) / 32 - 1; c >= 0; --c) {
+    int best = -1;
+    for (int sd = 0; sd < 4; ++sd) {
+      if (wave_n[sd] >= 2 && wave_n[sd + 4] >= 2) continue;
+      if (best < 0 || wave_load[sd] + wave_load[sd + 4] < wave_load[best] + wave_load[best + 4])
+        best = sd;
+    }
+    int w = best;
+    if (wave_n[w] >= 2 || (wave_n[w + 4] < 2 && wave_load[w + 4] < wave_load[w])) w = best + 4;
+    p.chunk[w][wave_n[w]++] = (signed char)c;
+    wave_load[w] += c + 1;
+  }
+  return p;
+}
+
 constexpr int RESIDENT_WAVES = 8;
 
 // LDS bytes of the resident variant, or 0 if this (L, D) does not fit two workgroups per CU.
@@ -627,6 +986,46 @@ int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t
   return 0;
 }
 
+// CUs of the current device, or a negative error code.
+inline int attn_cu_count() {
+  static int num_cus = 0;  // idempotent one-time setup; a race only repeats it
+  if (num_cus == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus < 1) {
+      set_error("flash_attn: cannot query the CU count");
+      return -4;
+    }
+    num_cus = cus;
+  }
+  return num_cus;
+}
+
+template <bool BLND>
+int launch_stream_attn(const void* q, const void* k, const void* v, void* out, int64_t BN,
+                       int heads, int L, float scale, hipStream_t st) {
+  auto kern = flash_attn_stream_kernel<BLND>;
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(160 KB LDS): %s", hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  const int cus = attn_cu_count();
+  if (cus < 0) return cus;
+  const int Lp = (L + BKEY - 1) / BKEY * BKEY;
+  const int grid = BN < cus ? (int)BN : cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), (size_t)Lp * 512, st,
+                     (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (_Float16*)out,
+                     heads, L, (int)BN, scale, make_stream_plan(L));
+  return 0;
+}
+
 template <int D, typename T>
 int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
              int heads, int L, float scale, Dropout drop, bool blnd, hipStream_t st) {
@@ -634,6 +1033,13 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
   if (drop.p > 0.f) {  // training-mode path: the tiled kernel carries the generator
     return blnd ? launch_tiled<D, T, true, true>(q, k, v, out, BN, heads, L, scale, da, st)
                 : launch_tiled<D, T, false, true>(q, k, v, out, BN, heads, L, scale, da, st);
+  }
+  if constexpr (D == 64 && sizeof(T) == 2) {
+    // fp16, head size 64, two (batch, head) pairs fit the LDS, enough pairs to keep every
+    // persistent workgroup busy for a while: the streaming kernel
+    if (L <= 320 && BN >= 64)
+      return blnd ? launch_stream_attn<true>(q, k, v, out, BN, heads, L, scale, st)
+                  : launch_stream_attn<false>(q, k, v, out, BN, heads, L, scale, st);
   }
   if (const size_t lds = resident_lds_bytes(L, D)) {
     return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
