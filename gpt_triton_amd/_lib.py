@@ -19,6 +19,8 @@ SIGNATURES = {
     "gptmi_last_error": (ctypes.c_char_p, []),
     "gptmi_embed": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _u64, _int,
                            _vp]),
+    "gptmi_embed_layernorm": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                     _i64, _f32, _int, _vp]),
     "gptmi_layernorm": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _int, _vp]),
     "gptmi_softmax": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "gptmi_linear_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),

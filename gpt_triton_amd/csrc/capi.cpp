@@ -215,6 +215,35 @@ int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
   return check_launch("embed");
 }
 
+int gptmi_embed_layernorm(const int64_t* ids, const void* wte, const void* wpe,
+                          const void* ln_w, const void* ln_b, void* emb, void* out, int64_t B,
+                          int64_t L, int64_t V, int64_t P, int64_t H, float eps, int dtype,
+                          void* stream) {
+  if (!ids || !wte || !wpe || !ln_w || !ln_b || !emb || !out || B <= 0 || L <= 0 || V <= 0 ||
+      P <= 0 || H <= 0 || !dtype_ok(dtype)) {
+    set_error("embed_layernorm: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (L > P) {
+    set_error("embed_layernorm: sequence length %lld exceeds the %lld position rows",
+              (long long)L, (long long)P);
+    return GPTMI_ERR_INVALID;
+  }
+  if (H > 8192) {
+    set_error("embed_layernorm: H=%lld beyond the supported 8192", (long long)H);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  const bool f16 = dtype == GPTMI_F16;
+  hipStream_t st = (hipStream_t)stream;
+  if (!launch_embed_layernorm(ids, wte, wpe, ln_w, ln_b, emb, out, B * L, L, V, (int)H, eps, f16,
+                              st)) {
+    // rows the fused kernel does not hold in registers: the two kernels, same results
+    launch_embed(ids, wte, wpe, emb, B * L, L, V, (int)H, Dropout{0.0f, 1337}, f16, st);
+    launch_layernorm(emb, ln_w, ln_b, out, B * L, (int)H, eps, f16, st);
+  }
+  return check_launch("embed_layernorm");
+}
+
 int gptmi_layernorm(const void* x, const void* w, const void* b, void* out, int64_t M,
                     int64_t H, float eps, int dtype, void* stream) {
   if (!x || !w || !b || !out || M <= 0 || H <= 0 || !dtype_ok(dtype)) {

@@ -14,6 +14,9 @@ struct Dropout {
 
 int launch_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
                  int64_t rows, int64_t L, int64_t V, int H, Dropout drop, bool f16, hipStream_t st);
+bool launch_embed_layernorm(const int64_t* ids, const void* wte, const void* wpe, const void* w,
+                            const void* b, void* emb, void* out, int64_t rows, int64_t L,
+                            int64_t V, int H, float eps, bool f16, hipStream_t st);
 int launch_layernorm(const void* x, const void* w, const void* b, void* out,
                      int64_t M, int H, float eps, bool f16, hipStream_t st);
 int launch_softmax(const void* x, void* out, int64_t M, int H, bool f16,

@@ -84,6 +84,42 @@ __global__ __launch_bounds__(256) void embed_dropout_kernel(
   }
 }
 
+// The arithmetic of one LayerNorm row, shared by layernorm_vec_kernel and embed_layernorm_kernel
+// so that the two give the same bits: fp32 mean, then the centred biased variance, then
+// (x - mean) * rstd * w + b.  Contraction is spelled out (fmaf where a multiply-add is fused,
+// none elsewhere): left to the compiler, the two kernels were fused differently.
+#pragma clang fp contract(off)
+template <int CH, int VN, int LPR>
+__device__ __forceinline__ void layernorm_stats(const float (&v)[CH][VN], float s, int lane,
+                                                int nchunks, int H, float eps, float& mean,
+                                                float& rstd) {
+  mean = group_sum<LPR>(s) / (float)H;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    if (lane + i * LPR < nchunks) {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const float d = v[i][j] - mean;
+        q = __builtin_fmaf(d, d, q);
+      }
+    }
+  }
+  const float var = group_sum<LPR>(q) / (float)H;
+  rstd = 1.0f / sqrtf(var + eps);
+}
+__device__ __forceinline__ float layernorm_apply(float x, float mean, float rstd, float w, float b) {
+  const float z = (x - mean) * rstd;
+  float r = __builtin_fmaf(z, w, b);
+  // The result is an fp32 number that the caller rounds to the storage type (the reference's
+  // fp32 arithmetic followed by a cast).  Without this fence the compiler may merge the
+  // multiply-add and the conversion into one mixed-precision instruction that rounds the exact
+  // result once, straight to fp16 -- in some kernels and not in others.
+  asm("" : "+v"(r));
+  return r;
+}
+#pragma clang fp contract(fast)
+
 // ---------------------------------------------------------------------------
 // LayerNorm (reference: fused_layer_norm_kernel, kernels.py:104-145): fp32
 // mean, then fp32 centred biased variance, rstd = 1/sqrt(var + eps),
@@ -129,20 +165,8 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
       for (int j = 0; j < VN; ++j) v[i][j] = 0.f;
     }
   }
-  const float mean = group_sum<LPR>(s) / (float)H;
-  float q = 0.f;
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    if (lane + i * LPR < nchunks) {
-#pragma unroll
-      for (int j = 0; j < VN; ++j) {
-        const float d = v[i][j] - mean;
-        q += d * d;
-      }
-    }
-  }
-  const float var = group_sum<LPR>(q) / (float)H;
-  const float rstd = 1.0f / sqrtf(var + eps);
+  float mean, rstd;
+  layernorm_stats<CH, VN, LPR>(v, s, lane, nchunks, H, eps, mean, rstd);
   V* o = reinterpret_cast<V*>(out + row * H);
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
@@ -154,14 +178,74 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(
       }
       V to;
 #pragma unroll
-      for (int j = 0; j < VN; ++j) {
-        const float z = (v[i][j] - mean) * rstd;
-        to[j] = (T)(z * (float)tw[i][j] + (float)tb[i][j]);
-      }
+      for (int j = 0; j < VN; ++j)
+        to[j] = (T)layernorm_apply(v[i][j], mean, rstd, (float)tw[i][j], (float)tb[i][j]);
       // cached (not streaming) store: the [T, H] output is what the following GEMM reads, two
       // or three times over; it fits the 256 MB memory-side cache, and a GEMM fed from there
       // instead of HBM ran 12 % faster (its operand loads are only one k-tile ahead)
       o[c] = to;
+    }
+  }
+}
+
+// Embedding gather and the first LayerNorm in one pass: emb[row,:] = wte[id,:] + wpe[pos,:]
+// (rounded to the storage dtype, as embed_vec_kernel stores it) and ln[row,:] = LayerNorm of
+// that ROUNDED row, so both outputs are bit-identical to embed_vec_kernel followed by
+// layernorm_vec_kernel; the row never leaves the registers in between (fused_embeddings ->
+// fused_layer_norm in the reference, gpt.py:166-170 and 40).
+template <typename T, int CH, int LPR>
+__global__ __launch_bounds__(256) void embed_layernorm_kernel(
+    const int64_t* __restrict__ ids, const T* __restrict__ wte, const T* __restrict__ wpe,
+    const T* __restrict__ w, const T* __restrict__ b, T* __restrict__ emb, T* __restrict__ out,
+    int64_t rows, int64_t L, int64_t V_, int H, float eps) {
+  typedef typename Vec<T>::type V;
+  constexpr int VN = Vec<T>::N;
+  const int lane = threadIdx.x & (LPR - 1);
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+  if (row >= rows) return;
+  const int64_t tok = ids[row];
+  const bool known = (uint64_t)tok < (uint64_t)V_;
+  const int nchunks = H / VN;
+  const V* ar = reinterpret_cast<const V*>(wte + (known ? tok : 0) * H);
+  const V* pr = reinterpret_cast<const V*>(wpe + (row % L) * H);
+  const V* wv = reinterpret_cast<const V*>(w);
+  const V* bv = reinterpret_cast<const V*>(b);
+  V* eo = reinterpret_cast<V*>(emb + row * H);
+  float v[CH][VN];
+  V tw[CH], tb[CH];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * LPR;
+    if (c < nchunks) {
+      const V va = ar[c], vb = pr[c];
+      tw[i] = wv[c];
+      tb[i] = bv[c];
+      V e;
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        e[j] = (T)((known ? (float)va[j] : 0.f) + (float)vb[j]);
+        v[i][j] = (float)e[j];
+        s += v[i][j];
+      }
+      __builtin_nontemporal_store(e, eo + c);  // the residual stream; next read by a GEMM epilogue
+    } else {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) v[i][j] = 0.f;
+    }
+  }
+  float mean, rstd;
+  layernorm_stats<CH, VN, LPR>(v, s, lane, nchunks, H, eps, mean, rstd);
+  V* o = reinterpret_cast<V*>(out + row * H);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * LPR;
+    if (c < nchunks) {
+      V to;
+#pragma unroll
+      for (int j = 0; j < VN; ++j)
+        to[j] = (T)layernorm_apply(v[i][j], mean, rstd, (float)tw[i][j], (float)tb[i][j]);
+      o[c] = to;  // cached store, as in layernorm_vec_kernel: the following GEMM reads it
     }
   }
 }
@@ -426,6 +510,51 @@ int launch_softmax(const void* x, void* out, int64_t M, int H, bool f16,
                    hipStream_t st) {
   return f16 ? launch_softmax_t<_Float16>(x, out, M, H, st)
              : launch_softmax_t<float>(x, out, M, H, st);
+}
+
+template <typename T, int CH>
+static void eln_go(const int64_t* ids, const void* wte, const void* wpe, const void* w,
+                   const void* b, void* emb, void* out, int64_t rows, int64_t L, int64_t V, int H,
+                   float eps, int lpr, hipStream_t st) {
+  if (lpr == 32)
+    hipLaunchKernelGGL((embed_layernorm_kernel<T, CH, 32>), dim3((unsigned)((rows + 7) / 8)),
+                       dim3(256), 0, st, ids, (const T*)wte, (const T*)wpe, (const T*)w,
+                       (const T*)b, (T*)emb, (T*)out, rows, L, V, H, eps);
+  else
+    hipLaunchKernelGGL((embed_layernorm_kernel<T, CH, 64>), dim3((unsigned)((rows + 3) / 4)),
+                       dim3(256), 0, st, ids, (const T*)wte, (const T*)wpe, (const T*)w,
+                       (const T*)b, (T*)emb, (T*)out, rows, L, V, H, eps);
+}
+
+template <typename T>
+static bool launch_embed_layernorm_t(const int64_t* ids, const void* wte, const void* wpe,
+                                     const void* w, const void* b, void* emb, void* out,
+                                     int64_t rows, int64_t L, int64_t V, int H, float eps,
+                                     hipStream_t st) {
+  constexpr int VN = Vec<T>::N;
+  auto al = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+  if ((H % VN) != 0 || !al(wte) || !al(wpe) || !al(w) || !al(b) || !al(emb) || !al(out))
+    return false;
+  const int lpr = lanes_per_row(H / VN);
+  const int need = (H / VN + lpr - 1) / lpr;
+  if (need <= 1) eln_go<T, 1>(ids, wte, wpe, w, b, emb, out, rows, L, V, H, eps, lpr, st);
+  else if (need <= 2) eln_go<T, 2>(ids, wte, wpe, w, b, emb, out, rows, L, V, H, eps, lpr, st);
+  else if (need <= 3) eln_go<T, 3>(ids, wte, wpe, w, b, emb, out, rows, L, V, H, eps, lpr, st);
+  else if (need <= 4) eln_go<T, 4>(ids, wte, wpe, w, b, emb, out, rows, L, V, H, eps, lpr, st);
+  else return false;
+  return true;
+}
+
+// The fused embedding + LayerNorm launch for rows that fit the register-resident form (16-byte
+// aligned, at most 4 chunks per lane: H <= 2048 halves / 1024 floats); otherwise false, and
+// the caller launches the two kernels one after the other.
+bool launch_embed_layernorm(const int64_t* ids, const void* wte, const void* wpe, const void* w,
+                            const void* b, void* emb, void* out, int64_t rows, int64_t L,
+                            int64_t V, int H, float eps, bool f16, hipStream_t st) {
+  return f16 ? launch_embed_layernorm_t<_Float16>(ids, wte, wpe, w, b, emb, out, rows, L, V, H,
+                                                  eps, st)
+             : launch_embed_layernorm_t<float>(ids, wte, wpe, w, b, emb, out, rows, L, V, H, eps,
+                                               st);
 }
 
 void launch_pack_rows(const void* src, void* dst, int64_t R, int K, int Kp, bool f16,

@@ -21,8 +21,8 @@ from dataclasses import dataclass
 import torch
 import torch.nn as nn
 
-from .kernels import (flash_attention_v1, fused_embeddings, fused_ffn, fused_layer_norm, lm_head,
-                      matmul_and_split_qkv, pack_lm_head, pack_weight)
+from .kernels import (flash_attention_v1, fused_embeddings, fused_embeddings_layer_norm, fused_ffn,
+                      fused_layer_norm, lm_head, matmul_and_split_qkv, pack_lm_head, pack_weight)
 
 # dense fp16/bf16 tensor throughput, FLOP/s
 GPU_TO_FLOPS = {
@@ -90,10 +90,14 @@ class FusedAttention(nn.Module):
         self._packed.clear()
         return super().train(mode)
 
-    def forward(self, x):
+    def forward(self, x, normed=None):
+        """`normed`: LayerNorm(x) with this block's weights, if the caller already has it (the
+        first block of FusedGPT gets it from the embedding kernel)."""
         p = self.dropout_prob if self.training else 0.0
         skip = x
-        y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+        y = normed
+        if y is None:
+            y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
         q, k, v = matmul_and_split_qkv(y, self._weight("c_attn_weight"), self.c_attn_bias.data,
                                        self.num_heads)
         # [B, N, L, d] values in a [B, L, N, d] buffer: the head merge below copies nothing
@@ -192,8 +196,18 @@ class FusedGPT(nn.Module):
     def forward(self, x, return_logits=False):
         # causal by construction; no attention or padding mask is taken
         p = self.config.dropout if self.training else 0.0
-        x = fused_embeddings(x, self.wte_weight.data, self.wpe_weight.data, dropout_prob=p)
-        for block in self.blocks:
+        if p == 0.0 and len(self.blocks) > 0:
+            # eval mode: the first block's LayerNorm comes out of the embedding kernel
+            first = self.blocks[0]
+            x, y = fused_embeddings_layer_norm(x, self.wte_weight.data, self.wpe_weight.data,
+                                               first[0].layer_norm_weight.data,
+                                               first[0].layer_norm_bias.data)
+            x = first[1](first[0](x, normed=y))
+            rest = self.blocks[1:]
+        else:
+            x = fused_embeddings(x, self.wte_weight.data, self.wpe_weight.data, dropout_prob=p)
+            rest = self.blocks
+        for block in rest:
             x = block(x)
         x = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
         if return_logits:

@@ -9,7 +9,8 @@ pointers to one entry point of libgptmi.so (include/gptmi.h).
     matmul_and_split_qkv(x, weight, bias, num_heads)             kernels.py:347-367
     flash_attention_v1(q, k, v, dropout_prob=0.0)                kernels.py:477-525
 
-plus `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:318-342),
+plus `fused_embeddings_layer_norm` (the embedding gather and the first block's LayerNorm in one
+kernel, the fusion the reference's author notes as a TODO, kernels.py:132-133), `fused_softmax(x)` (the reference only sketches a row softmax, kernels.py:318-342),
 `lm_head(x, wte)` (the transposed-weight product the reference leaves as a TODO,
 gpt.py:159-161) and `pack_weight(weight)`: the GEMM reads its weight as an fp16,
 K-contiguous image which `fused_ffn` / `matmul_and_split_qkv` otherwise rebuild on every
@@ -139,6 +140,39 @@ def fused_embeddings(x, wte, wpe, dropout_prob=0.0):
                              _stream())
     _lib.check(rc, "fused_embeddings")
     return z.view((B, L, H))
+
+
+@torch.no_grad()
+def fused_embeddings_layer_norm(x, wte, wpe, weight, bias):
+    """(fused_embeddings(x, wte, wpe), fused_layer_norm(of that, weight, bias)) from one kernel:
+    the embedding row is normalised while it is still in registers.  Both results are
+    bit-identical to the two separate calls.  No dropout (eval-mode forward)."""
+    assert wte.shape[1] == wpe.shape[1]
+    assert x.is_contiguous()
+    assert wte.is_contiguous()
+    assert wpe.is_contiguous()
+    assert weight.is_contiguous()
+    assert bias.is_contiguous()
+    assert weight.shape == bias.shape
+    assert wte.shape[1] == weight.shape[0]
+    B, L = x.shape
+    V, H = wte.shape
+    P = wpe.shape[0]
+    if x.dtype != torch.int64:
+        raise TypeError(f"fused_embeddings_layer_norm: token ids must be int64, got {x.dtype}")
+    if not (wte.dtype == wpe.dtype == weight.dtype == bias.dtype):
+        raise TypeError("fused_embeddings_layer_norm: wte, wpe, weight and bias must share a dtype")
+    dev = _on_gpu(x, wte, wpe, weight, bias)
+    emb = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
+    out = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_embed_layernorm(x.data_ptr(), wte.data_ptr(), wpe.data_ptr(),
+                                       weight.data_ptr(), bias.data_ptr(), emb.data_ptr(),
+                                       out.data_ptr(), B, L, V, P, H, 1e-5,
+                                       _dtype_code(wte, "fused_embeddings_layer_norm"), _stream())
+    _lib.check(rc, "fused_embeddings_layer_norm")
+    return emb.view((B, L, H)), out.view((B, L, H))
 
 
 @torch.no_grad()

@@ -87,6 +87,22 @@ int gptmi_embed(const int64_t* ids, const void* wte, const void* wpe, void* out,
                 float p, uint64_t seed, int dtype, void* stream);
 
 /*
+ * gptmi_embed (without dropout) and gptmi_layernorm of its result in one pass over the rows:
+ *   emb[b,l,:] = wte[ids[b,l],:] + wpe[l,:]          out[b,l,:] = LayerNorm(emb[b,l,:]; ln_w, ln_b)
+ * Both outputs are bit-identical to the two calls made one after the other (the LayerNorm works
+ * on the sum as rounded to the storage dtype); the row stays in registers in between.
+ *
+ * Replaces the pair fused_embeddings(x, wte, wpe) -> gpt.py:166-170 / kernels.py:75-101 and the
+ * first block's fused_layer_norm(x, weight, bias) -> gpt.py:40 / kernels.py:148-164, which the
+ * reference's author marks as a fusion to do (kernels.py:132-133).
+ *   ids int64 [B*L]   wte [V][H]   wpe [P][H]   ln_w, ln_b [H]   emb, out [B*L][H]   H <= 8192
+ */
+int gptmi_embed_layernorm(const int64_t* ids, const void* wte, const void* wpe,
+                          const void* ln_w, const void* ln_b, void* emb, void* out,
+                          int64_t B, int64_t L, int64_t V, int64_t P, int64_t H, float eps,
+                          int dtype, void* stream);
+
+/*
  * out[m,:] = (x[m,:] - mean_m) * rstd_m * w + b, rstd = 1/sqrt(var + eps),
  * mean and the centred, biased variance in fp32; x is read from HBM once.
  *

@@ -154,6 +154,35 @@ def test_fused_embeddings_out_of_range_ids_read_nothing(K, gpu_device):
         assert np.array_equal(host(z), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("H", [768, 1600, 256, 33, 4096])
+def test_fused_embeddings_layer_norm_equals_the_two_calls(K, gpu_device, dtype, H):
+    """The embedding gather with the first LayerNorm fused in (the reference author's TODO,
+    kernels.py:132-133): both outputs bit-identical to fused_embeddings followed by
+    fused_layer_norm, for widths the fused kernel holds in registers (768, 1600, 256) and widths
+    it hands to the two kernels (33: unaligned rows, 4096: too long), and against the oracle."""
+    r = np.random.default_rng(H)
+    V, P, B, L = 997, 40, 5, 37
+    ids = r.integers(0, V, size=(B, L))
+    ids[0, 0] = V + 5  # out of range: the row is the position embedding
+    wte = r.standard_normal((V, H)).astype(NP[dtype])
+    wpe = r.standard_normal((P, H)).astype(NP[dtype])
+    w = (1 + 0.1 * r.standard_normal(H)).astype(NP[dtype])
+    b = (0.1 * r.standard_normal(H)).astype(NP[dtype])
+    D = lambda a: dev(a, gpu_device)
+    emb, ln = K.fused_embeddings_layer_norm(D(ids), D(wte), D(wpe), D(w), D(b))
+    emb2 = K.fused_embeddings(D(ids), D(wte), D(wpe))
+    ln2 = K.fused_layer_norm(emb2, D(w), D(b))
+    assert emb.shape == ln.shape == (B, L, H)
+    assert torch.equal(emb, emb2) and torch.equal(ln, ln2)
+    ok = ids.copy()
+    ok[0, 0] = 0
+    want_e = O.fused_embeddings(ok, wte, wpe)
+    want_e[0, 0] = wpe[0]
+    assert np.array_equal(host(emb), want_e)
+    check(host(ln), O.fused_layer_norm(want_e, w, b), dtype, "fused embedding + layer norm")
+
+
 # ----------------------------------------------------------------------------- layer norm
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("M", [249, 32])
