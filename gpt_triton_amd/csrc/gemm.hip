@@ -167,6 +167,40 @@ __device__ __forceinline__ T* qkv_column_base(const EpiDev& ep, int n) {
   return base + ((int64_t)head * ep.L * ep.d + dd);
 }
 
+// Bias of a wavefront's columns in the accumulator layout: [i][g] -> the 4 consecutive columns
+// nw0 + 32 i + 8 g + 4 fhalf + 0..3, as stored (load_bias) and as fp32 (bias_to_f32).  ONE branch
+// stands around all the loads: with a test of ep.bias per load, every load got a basic block of
+// its own and, behind it, a wait for everything in flight -- 8 memory round trips per tile, one
+// after the other.  Needs 4-element vector access (N % 4 == 0, aligned bias: EpiDev::vec_ok).
+template <typename T, int NB>
+__device__ __forceinline__ void load_bias(const EpiDev& ep, int nw0, int fhalf,
+                                          typename Pack4<T>::type (&raw)[NB][4]) {
+  typedef typename Pack4<T>::type P4;
+  if (ep.bias) {
+    const T* bp = (const T*)ep.bias + (nw0 + fhalf * 4);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) raw[i][g] = *reinterpret_cast<const P4*>(bp + i * 32 + g * 8);
+  } else {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) raw[i][g][e] = 0;
+  }
+}
+template <typename P4, int NB>
+__device__ __forceinline__ void bias_to_f32(const P4 (&raw)[NB][4], f4 (&bias_r)[NB][4]) {
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bias_r[i][g][e] = (float)raw[i][g][e];
+}
+
 constexpr int EP_STRIDE = 64 * 4 + 16;  // bytes of one staged epilogue row (64 fp32 + pad)
 constexpr int EP_SLAB = 32 * EP_STRIDE; // one wavefront's staging slab
 
@@ -190,26 +224,26 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
 
   // bias of this lane's columns, fetched once: [i][g] -> 4 consecutive columns
   f4 bias_r[NB][4];
+  if constexpr (FAST) {
+    P4 raw[NB][4];
+    load_bias<T, NB>(ep, nw0, fhalf, raw);
+    bias_to_f32(raw, bias_r);
+  } else {
 #pragma unroll
-  for (int i = 0; i < NB; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
-      f4 b = {0.f, 0.f, 0.f, 0.f};
-      if (ep.bias) {
-        const T* bp = (const T*)ep.bias + n;
-        if (FAST) {
-          const P4 t = *reinterpret_cast<const P4*>(bp);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-        } else {
+      for (int g = 0; g < 4; ++g) {
+        const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
+        f4 b = {0.f, 0.f, 0.f, 0.f};
+        if (ep.bias) {
+          const T* bp = (const T*)ep.bias + n;
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (n + e < N) b[e] = (float)bp[e];
         }
+        bias_r[i][g] = b;
       }
-      bias_r[i][g] = b;
-    }
+  }
 
   // head-major scatter: the column part of the address once per 64-column slab, the row part
   // (b, l) = divmod(m, L) once for the lane's first row and then by stepping -- the sub-tile
@@ -450,6 +484,61 @@ __device__ __forceinline__ void store_wave_tile_rl(f16v (&acc)[NB][MB], const f4
   }
 }
 
+// store_wave_tile_rl for the streaming residual kernel.  The residual halves lie in the two
+// operand stages; `mid` runs between row bands 1 and 2, when the stage that held the first half
+// is free again (the kernel refills it there).  Younger than the first half's loads when band 0
+// starts: the second half's 8 loads.  Younger than the second half's loads when band 2 starts: the
+// 8 stores of bands 0 and 1 and, if `refilled`, the 8 operand loads `mid` issued.
+template <int MB, int NB, bool GELU, typename Mid>
+__device__ __forceinline__ void store_wave_tile_rs(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
+                                                   const char* res_lo, const char* res_hi,
+                                                   char* slab, int lane, bool refilled, Mid&& mid) {
+  static_assert(MB == 4 && NB == 2, "128 x 64 sub-tile");
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int rrow = lane >> 3, runit = lane & 7, rkey = rrow >> 1;
+  const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+    if (j == 0) wait_vmcnt<8>();
+    if (j == 2) {
+      mid();
+      if (refilled) wait_vmcnt<16>();
+      else wait_vmcnt<8>();
+    }
+    const char* rb = (j < 2 ? res_lo : res_hi) + ((j & 1) * 32 + frow) * 128 + fhalf * 8;
+    h4 r[NB][4];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        r[i][g] = *reinterpret_cast<const h4*>(rb + (((i * 4 + g) ^ fkey) << 4));
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        h4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          if (GELU) z = gelu_new(z);
+          o[e] = (_Float16)(z + (float)r[i][g][e]);
+        }
+        *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+      }
+    h8 vv[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+      vv[rr] = *reinterpret_cast<const h8*>(slab + (rr * 8 + rrow) * 128 +
+                                            ((runit ^ rkey ^ ((rr & 1) * 4)) << 4));
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+      store_nt_base(reinterpret_cast<char*>(ep.out) +
+                        ((mw0 + j * 32 + rr * 8) * (int64_t)N + nw0) * 2,
+                    lane_byte_off, vv[rr]);
+  }
+}
+
 template <int MB, int NB, typename T, bool QKV>
 __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDev& ep,
                                                 int64_t mw0, int nw0, int M, int N, bool fast,
@@ -468,20 +557,10 @@ __device__ __forceinline__ void store_wave_tile(f16v (&acc)[NB][MB], const EpiDe
   if constexpr (sizeof(T) == 2) {
     if (fast && !res && ep.vec8_ok) {
       const int fhalf = lane >> 5;
+      h4 raw[NB][4];
       f4 bias_r[NB][4];
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f4 b = {0.f, 0.f, 0.f, 0.f};
-          if (ep.bias) {
-            const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
-                                                       (nw0 + i * 32 + g * 8 + fhalf * 4));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-          }
-          bias_r[i][g] = b;
-        }
+      load_bias<_Float16, NB>(ep, nw0, fhalf, raw);
+      bias_to_f32(raw, bias_r);
       if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       else store_wave_tile_h<MB, NB, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       return;
@@ -723,20 +802,10 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       const int nw0 = n0 + wn * TN, fhalf = lane >> 5;
       // the bias first, and waited for, so that no compiler-placed wait inside the epilogue
       // falls behind the second half's loads
+      h4 raw[NB][4];
       f4 bias_r[NB][4];
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f4 b = {0.f, 0.f, 0.f, 0.f};
-          if (ep.bias) {
-            const h4 t = *reinterpret_cast<const h4*>((const _Float16*)ep.bias +
-                                                       (nw0 + i * 32 + g * 8 + fhalf * 4));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-          }
-          bias_r[i][g] = b;
-        }
+      load_bias<_Float16, NB>(ep, nw0, fhalf, raw);
+      bias_to_f32(raw, bias_r);
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
@@ -1038,29 +1107,22 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     }
 
     // last k-tile: before its final slice the next tile's first k-tile is published (this
-    // stage is free for a refill then); the bias is fetched and waited for BEFORE the next
-    // tile's second k-tile is requested, so that no wait inside the epilogue falls behind those
-    // loads.  The next tile's first fragments are read after the epilogue (registers).
+    // stage is free for a refill then); the bias is requested in front of the k-tile and waited
+    // for BEFORE the next tile's second k-tile is requested, so that no wait inside the epilogue
+    // falls behind those loads.  The next tile's first fragments are read after the epilogue.
+    // fp16: requested a whole k-tile before it is needed; fp32 (twice the registers): in front
+    // of the last slice
+    typename Pack4<T>::type bias_raw[NB][4];
+    if constexpr (sizeof(T) == 2) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+    __builtin_amdgcn_sched_barrier(0);
     first_slices();
     if (has_next) publish_next(false, false);
-    f4 bias_r[NB][4];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = nw0 + i * 32 + g * 8 + fhalf * 4;
-        f4 b = {0.f, 0.f, 0.f, 0.f};
-        if (ep.bias) {
-          const typename Pack4<T>::type t =
-              *reinterpret_cast<const typename Pack4<T>::type*>((const T*)ep.bias + n);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) b[e] = (float)t[e];
-        }
-        bias_r[i][g] = b;
-      }
+    if constexpr (sizeof(T) == 4) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
     __builtin_amdgcn_sched_barrier(0);
     mma(1);
     __builtin_amdgcn_sched_barrier(0);
+    f4 bias_r[NB][4];
+    bias_to_f32(bias_raw, bias_r);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
@@ -1082,6 +1144,241 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     if (!has_next) break;
     read_frags(stage, 0, 0);
     first_tile = false;
+    vp = vp_next;
+    m0 = m0_n;
+    n0 = n0_n;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Streaming kernel WITH a residual (fp16 row-major output, whole 256 x 256 tiles): the
+// persistent pipeline of gemm_stream_kernel, and the residual brought through LDS as in
+// gemm_kernel<RESLDS>.  The residual of a tile (128 KB) has no place of its own in LDS, so it
+// takes the operand stages as they fall free at the end of the tile, and the next tile's first two
+// k-tiles take them back as the epilogue lets go of them:
+//
+//   final slice of k-tile KT-2   its stage is refilled with residual rows 0..63 of every
+//                                wavefront's 128 x 64 sub-tile (8 loads, dealt between the MFMAs)
+//   behind k-tile KT-1           barrier, then residual rows 64..127 into that stage (8 loads)
+//   epilogue, row bands 0, 1     read the first half, 8 stores
+//   between bands 1 and 2        barrier, then the NEXT tile's k-tile 0 into the first stage
+//   epilogue, row bands 2, 3     read the second half, 8 stores
+//   behind the epilogue          barrier, then the next tile's k-tile 1 into the second stage
+//   start of the next tile       k-tile 0 has landed when at most 16 operations are outstanding
+//                                (8 stores and 8 loads are younger), barrier, first fragments
+//
+// A barrier stands in front of every refill because a wavefront's loads write stripes of every
+// wavefront's part of a stage.  What this buys over one workgroup per tile: no pipeline fill per
+// tile beyond what the epilogue's second half hides, and no idle CU between two workgroups while
+// the stores of the one that ended drain.  Whole tiles only; the launcher sends row tiles that
+// do not fill a round of the persistent workgroups to the small-tile kernel.
+// ---------------------------------------------------------------------------
+template <int WM, int WN>
+__global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
+    const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
+    int tiles_m, int tiles_n, int group_w, EpiDev ep) {
+  constexpr int BM = 256, BN = 256, ROWB = 128, T_ = 512, KS = 4;
+  static_assert(WM == 2 && WN == 4, "8 wavefronts, 128 x 64 sub-tiles");
+  constexpr int TM = BM / WM, TN = BN / WN;
+  constexpr int MB = TM / 32, NB = TN / 32;
+  constexpr int A_IT = 4, B_IT = 4, LPT = A_IT + B_IT;
+  constexpr int STAGE = (BM + BN) * ROWB;  // 64 KB
+  constexpr int SLABS = 2 * STAGE;
+  static_assert(MB * NB == LPT, "one load per MFMA of a k-slice");
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  const int num_tiles = tiles_m * tiles_n;
+  const int KT = Kp / 64;  // >= 2 (checked by the launcher)
+
+  const int r0 = tid >> 3;
+  unsigned lane_off[A_IT];
+#pragma unroll
+  for (int it = 0; it < A_IT; ++it)
+    lane_off[it] = (unsigned)(r0 + it * 64) * (unsigned)Kp * 2u +
+                   (unsigned)(((tid & 7) ^ ((r0 >> 1) & 7)) * 16);
+  const unsigned smem_base = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem);
+  const unsigned wave_off = smem_base + (unsigned)wave * 1024u;
+  auto tile_origin = [&](int vp, int& m0, int& n0) {
+    const int tile = xcd_tile(vp, num_tiles);
+    const int grp = tile / (tiles_m * group_w);
+    const int in_grp = tile - grp * tiles_m * group_w;
+    const int grp_w = min(group_w, tiles_n - grp * group_w);
+    m0 = (in_grp / grp_w) * BM;
+    n0 = (grp * group_w + in_grp % grp_w) * BN;
+  };
+  auto issue_one = [&](int stage, int m0, int n0, int k, int n) {
+    const unsigned base = wave_off + stage * STAGE;
+    if (n < A_IT)
+      lds_dma16_base((const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB), lane_off[n],
+                     base + n * T_ * 16);
+    else
+      lds_dma16_base((const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB),
+                     lane_off[n - A_IT], base + BM * ROWB + (n - A_IT) * T_ * 16);
+  };
+  auto issue = [&](int stage, int m0, int n0, int k) {
+#pragma unroll
+    for (int n = 0; n < LPT; ++n) issue_one(stage, m0, n0, k, n);
+  };
+  // Residual half h (rows 64 h .. 64 h + 63 of this wavefront's sub-tile) goes to the
+  // wavefront's own 8 KB of `stage`: load q fetches 8 rows, lane l the 16-byte unit
+  // (l % 8) ^ key of row 8 q + l / 8, key = (row >> 1) & 7 = (l / 16) ^ 4 (q & 1).
+  unsigned res_lane_off[2];
+#pragma unroll
+  for (int odd = 0; odd < 2; ++odd)
+    res_lane_off[odd] = ((unsigned)(lane >> 3) * (unsigned)N +
+                         (unsigned)(((lane & 7) ^ (lane >> 4) ^ (odd * 4)) * 8)) * 2u;
+  auto issue_res_one = [&](int stage, int m0, int n0, int h, int q) {
+    const char* base = (const char*)ep.residual +
+                       (((int64_t)m0 + wm * TM + h * 64 + q * 8) * N + (n0 + wn * TN)) * 2;
+    lds_dma16_base(base, res_lane_off[q & 1],
+                   smem_base + (unsigned)stage * STAGE + (unsigned)wave * 8192u + q * 1024);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int a_row_off = (wm * TM + frow) * ROWB;
+  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
+  h8 af[2][MB], bf[2][NB];
+  auto read_frags = [&](int stage, int ks, int slot) {
+    const char* st = smem + stage * STAGE;
+    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
+#pragma unroll
+    for (int j = 0; j < MB; ++j)
+      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
+  };
+  auto barrier_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  int vp = blockIdx.x;
+  int m0, n0;
+  tile_origin(vp, m0, n0);
+  issue(0, m0, n0, 0);
+  issue(1, m0, n0, 1);
+  wait_vmcnt<LPT>();
+  asm volatile("s_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+  int stage = 0;  // stage of the k-tile being multiplied
+
+  while (true) {
+    const int vp_next = vp + (int)gridDim.x;
+    const bool has_next = vp_next < num_tiles;
+    int m0_n = 0, n0_n = 0;
+    if (has_next) tile_origin(vp_next, m0_n, n0_n);
+    const int64_t mw0 = (int64_t)m0 + wm * TM;
+    const int nw0 = n0 + wn * TN;
+
+    f16v acc[NB][MB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < MB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    auto mma = [&](int slot) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
+                                                             0, 0, 0);
+    };
+    auto first_slices = [&]() {
+#pragma unroll
+      for (int ks = 0; ks < KS - 1; ++ks) {
+        read_frags(stage, ks + 1, (ks & 1) ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(ks & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+
+    // all k-tiles but the last: publish the next one (its loads are the only ones in flight),
+    // then the final slice refills this stage -- with the k-tile two ahead, or, behind the last
+    // but one, with the first half of the residual (that iteration is peeled off the loop)
+    auto publish_next = [&]() {
+      wait_vmcnt<0>();
+      barrier_lds();
+      read_frags(stage ^ 1, 0, 0);
+    };
+    for (int kt = 0; kt + 2 < KT; ++kt) {
+      first_slices();
+      publish_next();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
+          issue_one(stage, m0, n0, kt + 2, i * MB + j);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+      stage ^= 1;
+    }
+    {  // k-tile KT-2
+      first_slices();
+      publish_next();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
+          issue_res_one(stage, m0, n0, 0, i * MB + j);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+      stage ^= 1;
+    }
+
+    // last k-tile; behind its fragment reads the stage is free for the residual's second half.
+    // The bias is requested in front of the last slice and waited for behind it, before those
+    // loads are issued, so that no wait the compiler places falls behind them.
+    first_slices();
+    h4 bias_raw[NB][4];
+    load_bias<_Float16, NB>(ep, nw0, fhalf, bias_raw);  // all 8 loads in flight under the last slice
+    __builtin_amdgcn_sched_barrier(0);
+    mma(1);
+    __builtin_amdgcn_sched_barrier(0);
+    f4 bias_r[NB][4];
+    bias_to_f32(bias_raw, bias_r);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
+    barrier_lds();  // every wavefront has read the last k-tile's fragments
+#pragma unroll
+    for (int q = 0; q < 8; ++q) issue_res_one(stage, m0, n0, 1, q);
+    stage ^= 1;  // now the stage of k-tile KT-2: the residual's first half, then the next tile's k-tile 0
+
+    // ---- epilogue ----
+    {
+      const char* res_lo = smem + stage * STAGE + wave * 8192;
+      const char* res_hi = smem + (stage ^ 1) * STAGE + wave * 8192;
+      char* slab = smem + SLABS + wave * 4096;
+      auto mid = [&]() {
+        if (has_next) {
+          barrier_lds();  // nobody reads the first half any more
+          issue(stage, m0_n, n0_n, 0);
+        }
+      };
+      if (ep.gelu)
+        store_wave_tile_rs<MB, NB, true>(acc, bias_r, ep, mw0, nw0, N, res_lo, res_hi, slab, lane,
+                                         has_next, mid);
+      else
+        store_wave_tile_rs<MB, NB, false>(acc, bias_r, ep, mw0, nw0, N, res_lo, res_hi, slab, lane,
+                                          has_next, mid);
+    }
+    if (!has_next) break;
+    barrier_lds();  // nobody reads the second half any more
+    issue(stage ^ 1, m0_n, n0_n, 1);
+    // the next tile's k-tile 0: younger are the 8 stores of row bands 2 and 3 and the 8 loads above
+    wait_vmcnt<16>();
+    asm volatile("s_barrier" ::: "memory");
+    read_frags(stage, 0, 0);
     vp = vp_next;
     m0 = m0_n;
     n0 = n0_n;
@@ -1131,6 +1428,31 @@ int launch_stream(const void* A, const void* Bt, int64_t M, int N, int Kp, const
   return 0;
 }
 
+int launch_stream_res(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+                      hipStream_t st) {
+  auto kern = gemm_stream_res_kernel<2, 4>;
+  constexpr int smem = 2 * 512 * 128 + 8 * 4096;  // 160 KB: two stages + the epilogue slabs
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  const int num_cus = cu_count();
+  if (num_cus < 0) return num_cus;
+  const int tiles_m = (int)(M / 256), tiles_n = N / 256;
+  const int num_tiles = tiles_m * tiles_n;
+  const int group_w = column_group(tiles_n, 256, Kp);
+  const int grid = num_tiles < num_cus ? num_tiles : num_cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, st, (const _Float16*)A,
+                     (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n, group_w, ep);
+  return 0;
+}
+
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
@@ -1167,8 +1489,27 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     // fp16 with a residual, no dropout: whole tiles fetch the residual through LDS
     if constexpr (sizeof(T) == 2 && !QKV) {
       if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&
-          (((uintptr_t)ep.residual) & 15) == 0)
+          (((uintptr_t)ep.residual) & 15) == 0) {
+        if (M % 256 == 0 && N % 256 == 0 && Kp <= (1 << 21)) {
+          // whole tiles everywhere: the streaming kernel, with the same cut as above -- the row
+          // tiles that fill whole rounds of the persistent workgroups stay, the rest (headline
+          // N = 768: 1800 tiles = 7 rounds + 8; 597 of 600 row tiles stay) go to the small tiles
+          const int cus = cu_count();
+          if (cus < 0) return cus;
+          const int64_t tiles_m = M / 256, tiles_n = N / 256, tiles = tiles_m * tiles_n;
+          const int64_t rounds = tiles / cus, rem = tiles % cus;
+          int64_t m_head = M;
+          if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;
+          int rc = launch_stream_res(A, Bt, m_head, N, Kp, ep, st);
+          if (rc != 0 || m_head == M) return rc;
+          EpiDev tail = ep;
+          tail.out = (T*)ep.out + m_head * N;
+          tail.residual = (const T*)ep.residual + m_head * N;
+          return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>((const _Float16*)A + m_head * Kp, Bt,
+                                                              M - m_head, N, Kp, tail, st);
+        }
         return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV, true>(A, Bt, M, N, Kp, ep, st);
+      }
     }
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }

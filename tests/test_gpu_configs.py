@@ -86,6 +86,40 @@ def test_headline_gemm_every_element(K, gpu_device, name, Kd, N, gelu, use_res, 
     assert_all_close_f16(z, want, name)
 
 
+@pytest.mark.parametrize("M,N,Kd,gelu,bias,in_place", [
+    (25600, 768, 128, False, True, False),    # 300 tiles: some workgroups walk two; 2 k-tiles
+    (25600, 768, 192, True, False, False),    # 3 k-tiles, GELU in front of the residual, no bias
+    (66560, 1024, 256, False, True, True),    # 1040 tiles = 4 rounds + 16: head + small-tile tail,
+                                              # output written over the residual
+    (4096, 768, 3072, False, True, False),    # 48 tiles: one each, nothing to refill
+])
+def test_residual_gemm_streaming_every_element(K, gpu_device, M, N, Kd, gelu, bias, in_place):
+    """fp16 GEMM + residual on whole 256 x 256 tiles (the persistent kernel that carries the
+    residual through the operand stages and refills them mid-epilogue): every element against the
+    fp32 torch product, NaN-poisoned output, k-tile counts 2, 3, 4 and 48, one or several tiles
+    per workgroup, with and without the small-tile tail, and in place."""
+    g = torch.Generator(device=gpu_device).manual_seed(M + Kd)
+    x = torch.randn((M, Kd), generator=g, device=gpu_device).half()
+    w = (torch.randn((Kd, N), generator=g, device=gpu_device) / Kd ** 0.5).half()
+    b = (0.1 * torch.randn(N, generator=g, device=gpu_device)).half() if bias else None
+    res = torch.randn((M, N), generator=g, device=gpu_device).half()
+    want = x.float() @ w.float()
+    if bias:
+        want = want + b.float()
+    if gelu:
+        want = gelu_tanh(want)
+    want = want + res.float()
+    print(f"residual streaming: M={M} N={N} K={Kd} gelu={gelu} bias={bias} in_place={in_place}",
+          flush=True)
+    if in_place:
+        z = res.clone()
+        K._linear(x, K.pack_weight(w), b, z, z, gelu, 0.0, K._lib.GPTMI_W_PACKED, "in place")
+    else:
+        z = torch.full((M, N), float("nan"), device=gpu_device, dtype=torch.float16)
+        K._linear(x, K.pack_weight(w), b, res, z, gelu, 0.0, K._lib.GPTMI_W_PACKED, "residual")
+    assert_all_close_f16(z, want, "residual streaming")
+
+
 def test_headline_qkv_every_element(K, gpu_device):
     """The headline q/k/v product [153600, 768] @ [768, 2304] + b scattered head-major, every
     element of q, k and v, through gptmi_linear_qkv with NaN-poisoned outputs."""
