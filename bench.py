@@ -171,14 +171,20 @@ def bench_ops(dev):
     gemm = lambda n, k_: 2 * M * n * k_
     ops = [
         ("ffn1 768->3072 +bias+GELU", lambda: K.fused_ffn(x, w1, bias=b1, add_gelu=True), gemm(3072, 768), None, None),
+        # the same products with parts of the epilogue left out: the differences are what the
+        # bias, the GELU and the residual cost
+        ("ffn1 768->3072 +bias (no GELU)", lambda: K.fused_ffn(x, w1, bias=b1), gemm(3072, 768), None, None),
+        ("ffn1 768->3072 (no bias, no GELU)", lambda: K.fused_ffn(x, w1), gemm(3072, 768), None, None),
         ("ffn2 3072->768 +bias", lambda: K.fused_ffn(x4, w2, bias=b2), gemm(768, 3072), None, None),
         ("ffn2 3072->768 +bias+residual", lambda: K.fused_ffn(x4, w2, bias=b2, residual=x), gemm(768, 3072), None, None),
         ("qkv 768->2304 +bias, head-major split", lambda: K.matmul_and_split_qkv(x.view(BATCH, SEQLEN, h), wq, bq, 12), gemm(2304, 768), None, None),
         ("attention projection 768->768 +bias+residual", lambda: K.fused_ffn(x, wo, bias=bo, residual=x), gemm(768, 768), None, None),
+        ("attention projection 768->768 +bias (no residual)", lambda: K.fused_ffn(x, wo, bias=bo), gemm(768, 768), None, None),
         ("flash attention 512x12x300x64 causal", lambda: K.flash_attention_v1(q, k, v), 4 * BATCH * 12 * 64 * SEQLEN * (SEQLEN + 1) // 2, 4 * BATCH * 12 * SEQLEN * 64 * 2, flush),
         ("layernorm 153600x768", lambda: K.fused_layer_norm(x, lw, lb), None, 2 * M * h * 2, flush),
         ("softmax 153600x768", lambda: K.fused_softmax(x), None, 2 * M * h * 2, flush),
         ("embedding 512x300x768", lambda: K.fused_embeddings(ids, wte, wpe), None, M * 8 + 2 * M * h * 2 + SEQLEN * h * 2, flush),
+        ("embedding + first LayerNorm 512x300x768", lambda: K.fused_embeddings_layer_norm(ids, wte, wpe, lw, lb), None, M * 8 + 3 * M * h * 2 + SEQLEN * h * 2, flush),
     ]
     rows = []
     for name, fn, flops, nbytes, fl in ops:
