@@ -993,7 +993,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
                    (unsigned)(((tid & 7) ^ ((r0 >> 1) & 7)) * 16);
   const unsigned wave_off =
       __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + (unsigned)wave * 1024u);
-  auto tile_origin = [&](int vp, int& m0, int& n0) {
+  auto tile_origin = [&](int vp, int& m0, int& n0) __attribute__((always_inline)) {
     const int tile = xcd_tile(vp, num_tiles);
     const int grp = tile / (tiles_m * group_w);
     const int in_grp = tile - grp * tiles_m * group_w;
@@ -1001,26 +1001,35 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     m0 = (in_grp / grp_w) * BM;
     n0 = (grp * group_w + in_grp % grp_w) * BN;
   };
-  // load n (0..3: A, 4..7: B) of k-tile k of the tile at (m0, n0) into `stage`
-  auto issue_one = [&](int stage, int m0, int n0, int k, int n) {
-    const unsigned base = wave_off + stage * STAGE;
-    if (n < A_IT)
-      lds_dma16_base((const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB), lane_off[n],
-                     base + n * T_ * 16);
-    else
-      lds_dma16_base((const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB),
-                     lane_off[n - A_IT], base + BM * ROWB + (n - A_IT) * T_ * 16);
+  // A k-tile is eight 16-byte loads per lane: four for the A rows, four for the B rows.  The
+  // source of a half is a scalar (first row of the tile, first byte of the k-tile), computed once
+  // and not per load: the scalar work of a load that goes between two MFMAs must fit under one.
+  auto a_src = [&](int m0, int k) __attribute__((always_inline)) {
+    return (const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB);
   };
-  auto issue = [&](int stage, int m0, int n0, int k) {
+  auto b_src = [&](int n0, int k) __attribute__((always_inline)) {
+    return (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+  };
+  auto issue_a = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
+    lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + n * T_ * 16);
+  };
+  auto issue_b = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
+    lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + BM * ROWB + n * T_ * 16);
+  };
+  auto issue = [&](int stage, int m0, int n0, int k) __attribute__((always_inline)) {
+    const char* a = a_src(m0, k);
+    const char* b = b_src(n0, k);
 #pragma unroll
-    for (int n = 0; n < LPT; ++n) issue_one(stage, m0, n0, k, n);
+    for (int n = 0; n < A_IT; ++n) issue_a(stage, a, n);
+#pragma unroll
+    for (int n = 0; n < B_IT; ++n) issue_b(stage, b, n);
   };
 
   const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
   const int a_row_off = (wm * TM + frow) * ROWB;
   const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
   h8 af[2][MB], bf[2][NB];
-  auto read_frags = [&](int stage, int ks, int slot) {
+  auto read_frags = [&](int stage, int ks, int slot) __attribute__((always_inline)) {
     const char* st = smem + stage * STAGE;
     const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
@@ -1058,52 +1067,85 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    auto mma = [&](int slot) {
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
-                                                             0, 0, 0);
-    };
-    // k-slices 0..2 of the k-tile in `stage`: fragments of the next slice first, then the MFMAs
-    auto first_slices = [&]() {
-#pragma unroll
-      for (int ks = 0; ks < KS - 1; ++ks) {
-        read_frags(stage, ks + 1, (ks & 1) ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(ks & 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-    // publish the k-tile in the other stage and fetch its first fragments (slot 0)
-    auto publish_next = [&](bool behind_epilogue, bool fetch) {
-      // behind an epilogue exactly EPI_STORES stores are younger than the loads waited for
-      if (behind_epilogue) wait_vmcnt<EPI_STORES>();
-      else wait_vmcnt<0>();
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      if (fetch) read_frags(stage ^ 1, 0, 0);
-    };
-
-    // all k-tiles but the last: the final slice refills this stage with the k-tile two ahead
-    // (of this tile, or the first of the next one), the loads dealt between the MFMAs
-    for (int kt = 0; kt + 1 < KT; ++kt) {
-      first_slices();
-      publish_next(kt == 0 && !first_tile, true);
-      const bool own = kt + 2 < KT;
-      const bool go = own || has_next;
-      const int ra = own ? m0 : m0_n, rb = own ? n0 : n0_n;
-      const int kk = own ? kt + 2 : 0;
-      __builtin_amdgcn_sched_barrier(0);
+    // One k-slice: the eight MFMAs on fragment slot `slot`.  Behind the first six of them, one
+    // each, go the fragment reads of slice `rks` of `rstage` into the other slot, in the order
+    // the next slice uses them: a read issued in the shadow of an MFMA costs no issue time,
+    // six of them in front of the MFMAs idle the pipe whenever both wavefronts of a SIMD read
+    // at once (behind every barrier).  `extra(q)` runs behind MFMA q.
+    auto slice = [&](int slot, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+      const char* st = smem + rstage * STAGE;
+      const int choff = ((rks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int j = 0; j < MB; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
-          if (go) issue_one(stage, ra, rb, kk, i * MB + j);
+          const int q = i * MB + j;
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
+                                                             0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (fetch) {
+            if (q == 0)
+              bf[slot ^ 1][0] = *reinterpret_cast<const h8*>(st + b_row_off + choff);
+            else if (q <= MB)
+              af[slot ^ 1][q - 1] =
+                  *reinterpret_cast<const h8*>(st + a_row_off + (q - 1) * 32 * ROWB + choff);
+            else if (q < MB + NB)
+              bf[slot ^ 1][q - MB] =
+                  *reinterpret_cast<const h8*>(st + b_row_off + (q - MB) * 32 * ROWB + choff);
+          }
+          extra(q);
+          __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    auto nothing = [](int) __attribute__((always_inline)) {};
+    // A refill dealt one load behind every MFMA of one slice arrives at the texture unit faster
+    // than it takes them (64 loads per CU in the time of 16 MFMAs): the wavefronts stall on
+    // issue, the MFMAs behind the loads too.  So the A half goes behind every second MFMA of the
+    // slice that frees the stage and the B half behind every second MFMA of the next slice.
+    const char* b_half = nullptr;  // B half still to be issued into the other stage
+    auto with_b_half = [&](int q) __attribute__((always_inline)) {
+      if (q & 1) issue_b(stage ^ 1, b_half, q / 2);
+    };
+    // k-slices 0..2 of the k-tile in `stage`; `extra0` goes with the first
+    auto first_slices = [&](auto&& extra0) __attribute__((always_inline)) {
+      slice(0, true, stage, 1, extra0);
+      slice(1, true, stage, 2, nothing);
+      slice(0, true, stage, 3, nothing);
+    };
+    // publish the k-tile in the other stage
+    auto publish_next = [&](bool behind_epilogue) __attribute__((always_inline)) {
+      // behind an epilogue exactly EPI_STORES stores are younger than the loads waited for
+      if (behind_epilogue) wait_vmcnt<EPI_STORES>();
+      else wait_vmcnt<0>();
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    // The final slice of k-tile kt (not the last): it takes the first fragments of the published
+    // k-tile and starts the refill of this stage with the k-tile two ahead -- of this tile, or
+    // the first of the next one; behind the last tile it loads this tile's first k-tile again,
+    // which nobody reads (no branch around the loads).
+    auto final_slice = [&](int kt) __attribute__((always_inline)) {
+      const bool own = kt + 2 < KT;
+      // (values, not a choice between two captured variables: that would index the closure)
+      const bool stay = own || !has_next;
+      const int ra = stay ? +m0 : +m0_n, rb = stay ? +n0 : +n0_n;
+      const int kk = own ? kt + 2 : 0;
+      const char* src = a_src(ra, kk);
       __builtin_amdgcn_sched_barrier(0);
+      slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
+        if (q & 1) issue_a(stage, src, q / 2);
+      });
+      b_half = b_src(rb, kk);
       stage ^= 1;
+    };
+
+    // all k-tiles but the last; the first has no half refill to carry
+    first_slices(nothing);
+    publish_next(!first_tile);
+    final_slice(0);
+    for (int kt = 1; kt + 1 < KT; ++kt) {
+      first_slices(with_b_half);
+      publish_next(false);
+      final_slice(kt);
     }
 
     // last k-tile: before its final slice the next tile's first k-tile is published (this
@@ -1115,12 +1157,11 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     typename Pack4<T>::type bias_raw[NB][4];
     if constexpr (sizeof(T) == 2) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
     __builtin_amdgcn_sched_barrier(0);
-    first_slices();
-    if (has_next) publish_next(false, false);
+    first_slices(with_b_half);
+    if (has_next) publish_next(false);
     if constexpr (sizeof(T) == 4) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
     __builtin_amdgcn_sched_barrier(0);
-    mma(1);
-    __builtin_amdgcn_sched_barrier(0);
+    slice(1, false, 0, 0, nothing);
     f4 bias_r[NB][4];
     bias_to_f32(bias_raw, bias_r);
 #pragma unroll
@@ -1148,6 +1189,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     m0 = m0_n;
     n0 = n0_n;
   }
+  wait_vmcnt<0>();  // the last tile's unread refill
 }
 
 // ---------------------------------------------------------------------------
@@ -1191,7 +1233,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % WM, wn = wave / WM;
   const int num_tiles = tiles_m * tiles_n;
-  const int KT = Kp / 64;  // >= 2 (checked by the launcher)
+  const int KT = Kp / 64;  // >= 3 (checked by the launcher)
 
   const int r0 = tid >> 3;
   unsigned lane_off[A_IT];
@@ -1201,7 +1243,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
                    (unsigned)(((tid & 7) ^ ((r0 >> 1) & 7)) * 16);
   const unsigned smem_base = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem);
   const unsigned wave_off = smem_base + (unsigned)wave * 1024u;
-  auto tile_origin = [&](int vp, int& m0, int& n0) {
+  auto tile_origin = [&](int vp, int& m0, int& n0) __attribute__((always_inline)) {
     const int tile = xcd_tile(vp, num_tiles);
     const int grp = tile / (tiles_m * group_w);
     const int in_grp = tile - grp * tiles_m * group_w;
@@ -1209,18 +1251,27 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     m0 = (in_grp / grp_w) * BM;
     n0 = (grp * group_w + in_grp % grp_w) * BN;
   };
-  auto issue_one = [&](int stage, int m0, int n0, int k, int n) {
-    const unsigned base = wave_off + stage * STAGE;
-    if (n < A_IT)
-      lds_dma16_base((const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB), lane_off[n],
-                     base + n * T_ * 16);
-    else
-      lds_dma16_base((const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB),
-                     lane_off[n - A_IT], base + BM * ROWB + (n - A_IT) * T_ * 16);
+  // the halves of a k-tile (four loads per lane each) and their scalar sources, as in
+  // gemm_stream_kernel
+  auto a_src = [&](int m0, int k) __attribute__((always_inline)) {
+    return (const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB);
   };
-  auto issue = [&](int stage, int m0, int n0, int k) {
+  auto b_src = [&](int n0, int k) __attribute__((always_inline)) {
+    return (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+  };
+  auto issue_a = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
+    lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + n * T_ * 16);
+  };
+  auto issue_b = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
+    lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + BM * ROWB + n * T_ * 16);
+  };
+  auto issue = [&](int stage, int m0, int n0, int k) __attribute__((always_inline)) {
+    const char* a = a_src(m0, k);
+    const char* b = b_src(n0, k);
 #pragma unroll
-    for (int n = 0; n < LPT; ++n) issue_one(stage, m0, n0, k, n);
+    for (int n = 0; n < A_IT; ++n) issue_a(stage, a, n);
+#pragma unroll
+    for (int n = 0; n < B_IT; ++n) issue_b(stage, b, n);
   };
   // Residual half h (rows 64 h .. 64 h + 63 of this wavefront's sub-tile) goes to the
   // wavefront's own 8 KB of `stage`: load q fetches 8 rows, lane l the 16-byte unit
@@ -1230,10 +1281,13 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   for (int odd = 0; odd < 2; ++odd)
     res_lane_off[odd] = ((unsigned)(lane >> 3) * (unsigned)N +
                          (unsigned)(((lane & 7) ^ (lane >> 4) ^ (odd * 4)) * 8)) * 2u;
-  auto issue_res_one = [&](int stage, int m0, int n0, int h, int q) {
-    const char* base = (const char*)ep.residual +
-                       (((int64_t)m0 + wm * TM + h * 64 + q * 8) * N + (n0 + wn * TN)) * 2;
-    lds_dma16_base(base, res_lane_off[q & 1],
+  auto res_src = [&](int m0, int n0, int h) __attribute__((always_inline)) {
+    return (const char*)ep.residual +
+           (((int64_t)m0 + wm * TM + h * 64) * N + (n0 + wn * TN)) * 2;
+  };
+  const int64_t res_step = (int64_t)N * 16;  // 8 rows
+  auto issue_res_one = [&](int stage, const char* src, int q) __attribute__((always_inline)) {
+    lds_dma16_base(src + q * res_step, res_lane_off[q & 1],
                    smem_base + (unsigned)stage * STAGE + (unsigned)wave * 8192u + q * 1024);
   };
 
@@ -1241,7 +1295,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   const int a_row_off = (wm * TM + frow) * ROWB;
   const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
   h8 af[2][MB], bf[2][NB];
-  auto read_frags = [&](int stage, int ks, int slot) {
+  auto read_frags = [&](int stage, int ks, int slot) __attribute__((always_inline)) {
     const char* st = smem + stage * STAGE;
     const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
@@ -1251,7 +1305,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     for (int i = 0; i < NB; ++i)
       bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
   };
-  auto barrier_lds = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  auto barrier_lds = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   int vp = blockIdx.x;
   int m0, n0;
@@ -1279,70 +1333,94 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    auto mma = [&](int slot) {
+    // One k-slice, as in gemm_stream_kernel: eight MFMAs on fragment slot `slot`, the six
+    // fragment reads of slice `rks` of `rstage` behind the first six of them, `extra(q)` behind
+    // MFMA q.
+    auto slice = [&](int slot, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+      const char* st = smem + rstage * STAGE;
+      const int choff = ((rks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < MB; ++j)
+        for (int j = 0; j < MB; ++j) {
+          const int q = i * MB + j;
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
                                                              0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (fetch) {
+            if (q == 0)
+              bf[slot ^ 1][0] = *reinterpret_cast<const h8*>(st + b_row_off + choff);
+            else if (q <= MB)
+              af[slot ^ 1][q - 1] =
+                  *reinterpret_cast<const h8*>(st + a_row_off + (q - 1) * 32 * ROWB + choff);
+            else if (q < MB + NB)
+              bf[slot ^ 1][q - MB] =
+                  *reinterpret_cast<const h8*>(st + b_row_off + (q - MB) * 32 * ROWB + choff);
+          }
+          extra(q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
     };
-    auto first_slices = [&]() {
-#pragma unroll
-      for (int ks = 0; ks < KS - 1; ++ks) {
-        read_frags(stage, ks + 1, (ks & 1) ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(ks & 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    auto nothing = [](int) __attribute__((always_inline)) {};
+    // The three slices in front of a k-tile's last.  `extra0` deals the second half of the
+    // refill that the slice before started: four loads there, four here, because eight behind
+    // the MFMAs of one slice arrive faster than the texture unit takes them.
+    auto first_slices = [&](auto&& extra0) __attribute__((always_inline)) {
+      slice(0, true, stage, 1, extra0);
+      slice(1, true, stage, 2, nothing);
+      slice(0, true, stage, 3, nothing);
     };
-
-    // all k-tiles but the last: publish the next one (its loads are the only ones in flight),
-    // then the final slice refills this stage -- with the k-tile two ahead, or, behind the last
-    // but one, with the first half of the residual (that iteration is peeled off the loop)
-    auto publish_next = [&]() {
+    auto publish_next = [&]() __attribute__((always_inline)) {
       wait_vmcnt<0>();
       barrier_lds();
-      read_frags(stage ^ 1, 0, 0);
     };
-    for (int kt = 0; kt + 2 < KT; ++kt) {
-      first_slices();
-      publish_next();
+    const char* b_half = nullptr;  // B half still to be issued into the other stage
+    auto with_b_half = [&](int q) __attribute__((always_inline)) {
+      if (q & 1) issue_b(stage ^ 1, b_half, q / 2);
+    };
+    // the final slice of a k-tile in front of the last but one: it takes the first fragments of
+    // the published k-tile and starts the refill of this stage with the k-tile two ahead
+    auto final_slice = [&](int kt) __attribute__((always_inline)) {
+      const char* src = a_src(m0, kt + 2);
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
-          issue_one(stage, m0, n0, kt + 2, i * MB + j);
-        }
-      __builtin_amdgcn_sched_barrier(0);
+      slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
+        if (q & 1) issue_a(stage, src, q / 2);
+      });
+      b_half = b_src(n0, kt + 2);
       stage ^= 1;
-    }
-    {  // k-tile KT-2
-      first_slices();
-      publish_next();
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[1][i], af[1][j], acc[i][j], 0, 0, 0);
-          issue_res_one(stage, m0, n0, 0, i * MB + j);
-        }
-      __builtin_amdgcn_sched_barrier(0);
-      stage ^= 1;
-    }
+    };
 
-    // last k-tile; behind its fragment reads the stage is free for the residual's second half.
-    // The bias is requested in front of the last slice and waited for behind it, before those
-    // loads are issued, so that no wait the compiler places falls behind them.
-    first_slices();
+    // All k-tiles but the last two (KT >= 3, checked by the launcher): publish the next one (its
+    // loads are the only ones in flight), refill this stage.  The first has no half refill to
+    // carry.
+    first_slices(nothing);
+    publish_next();
+    final_slice(0);
+    for (int kt = 1; kt + 2 < KT; ++kt) {
+      first_slices(with_b_half);
+      publish_next();
+      final_slice(kt);
+    }
+    // k-tile KT-2: its stage takes the first half of the residual
+    const char* res0 = res_src(m0, n0, 0);
+    first_slices(with_b_half);
+    publish_next();
+    slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
+      if (q & 1) issue_res_one(stage, res0, q / 2);
+    });
+    stage ^= 1;
+
+    // last k-tile; its first slice carries the rest of the residual's first half, and behind its
+    // fragment reads the stage is free for the second half.  The bias is requested in front of
+    // the last slice and waited for behind it, before those loads are issued, so that no wait
+    // the compiler places falls behind them.
+    first_slices([&](int q) __attribute__((always_inline)) {
+      if (q & 1) issue_res_one(stage ^ 1, res0, 4 + q / 2);
+    });
     h4 bias_raw[NB][4];
     load_bias<_Float16, NB>(ep, nw0, fhalf, bias_raw);  // all 8 loads in flight under the last slice
     __builtin_amdgcn_sched_barrier(0);
-    mma(1);
-    __builtin_amdgcn_sched_barrier(0);
+    slice(1, false, 0, 0, nothing);
     f4 bias_r[NB][4];
     bias_to_f32(bias_raw, bias_r);
 #pragma unroll
@@ -1350,8 +1428,11 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
 #pragma unroll
       for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
     barrier_lds();  // every wavefront has read the last k-tile's fragments
+    {
+      const char* res1 = res_src(m0, n0, 1);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) issue_res_one(stage, m0, n0, 1, q);
+      for (int q = 0; q < 8; ++q) issue_res_one(stage, res1, q);
+    }
     stage ^= 1;  // now the stage of k-tile KT-2: the residual's first half, then the next tile's k-tile 0
 
     // ---- epilogue ----
@@ -1359,7 +1440,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
       const char* res_lo = smem + stage * STAGE + wave * 8192;
       const char* res_hi = smem + (stage ^ 1) * STAGE + wave * 8192;
       char* slab = smem + SLABS + wave * 4096;
-      auto mid = [&]() {
+      auto mid = [&]() __attribute__((always_inline)) {
         if (has_next) {
           barrier_lds();  // nobody reads the first half any more
           issue(stage, m0_n, n0_n, 0);
@@ -1490,8 +1571,8 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     if constexpr (sizeof(T) == 2 && !QKV) {
       if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&
           (((uintptr_t)ep.residual) & 15) == 0) {
-        if (M % 256 == 0 && N % 256 == 0 && Kp <= (1 << 21)) {
-          // whole tiles everywhere: the streaming kernel, with the same cut as above -- the row
+        if (M % 256 == 0 && N % 256 == 0 && Kp >= 192 && Kp <= (1 << 21)) {
+          // whole tiles everywhere and at least three k-tiles: the streaming kernel, with the same cut as above -- the row
           // tiles that fill whole rounds of the persistent workgroups stay, the rest (headline
           // N = 768: 1800 tiles = 7 rounds + 8; 597 of 600 row tiles stay) go to the small tiles
           const int cus = cu_count();
