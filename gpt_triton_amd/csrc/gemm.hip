@@ -1007,8 +1007,15 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   auto a_src = [&](int m0, int k) __attribute__((always_inline)) {
     return (const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB);
   };
-  auto b_src = [&](int n0, int k) __attribute__((always_inline)) {
-    return (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+  // Source of load n (64-row block n) of the B tile at n0.  N is a multiple of 64, not
+  // necessarily of 256: in the last column tile a block that starts at or past row N loads
+  // block 0 again (the shift goes into the scalar source, the lane offsets stay); its products
+  // are never stored.
+  const size_t blk_bytes = (size_t)64 * Kp * 2;
+  auto b_src = [&](int n0, int k, int n) __attribute__((always_inline)) {
+    const int vb = (N - n0) >> 6;  // valid blocks of this tile (4 or more: all)
+    const char* p = (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+    return n < vb ? p : p - n * blk_bytes;
   };
   auto issue_a = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
     lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + n * T_ * 16);
@@ -1018,11 +1025,10 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   };
   auto issue = [&](int stage, int m0, int n0, int k) __attribute__((always_inline)) {
     const char* a = a_src(m0, k);
-    const char* b = b_src(n0, k);
 #pragma unroll
     for (int n = 0; n < A_IT; ++n) issue_a(stage, a, n);
 #pragma unroll
-    for (int n = 0; n < B_IT; ++n) issue_b(stage, b, n);
+    for (int n = 0; n < B_IT; ++n) issue_b(stage, b_src(n0, k, n), n);
   };
 
   const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
@@ -1049,7 +1055,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   asm volatile("s_barrier" ::: "memory");
   read_frags(0, 0, 0);
   int stage = 0;           // stage of the k-tile being multiplied
-  bool first_tile = true;
+  bool prev_stored = false;  // this wavefront stored a tile right before the current one
 
   while (true) {
     const int vp_next = vp + (int)gridDim.x;
@@ -1058,6 +1064,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     if (has_next) tile_origin(vp_next, m0_n, n0_n);
     const int64_t mw0 = (int64_t)m0 + wm * TM;
     const int nw0 = n0 + wn * TN;
+    const bool wave_stores = nw0 < N;  // else this wavefront's 64 columns lie past the edge
 
     f16v acc[NB][MB];
 #pragma unroll
@@ -1102,9 +1109,9 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     // than it takes them (64 loads per CU in the time of 16 MFMAs): the wavefronts stall on
     // issue, the MFMAs behind the loads too.  So the A half goes behind every second MFMA of the
     // slice that frees the stage and the B half behind every second MFMA of the next slice.
-    const char* b_half = nullptr;  // B half still to be issued into the other stage
+    const char* b_half[B_IT] = {};  // B half still to be issued into the other stage
     auto with_b_half = [&](int q) __attribute__((always_inline)) {
-      if (q & 1) issue_b(stage ^ 1, b_half, q / 2);
+      if (q & 1) issue_b(stage ^ 1, b_half[q / 2], q / 2);
     };
     // k-slices 0..2 of the k-tile in `stage`; `extra0` goes with the first
     auto first_slices = [&](auto&& extra0) __attribute__((always_inline)) {
@@ -1134,13 +1141,14 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
       slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
         if (q & 1) issue_a(stage, src, q / 2);
       });
-      b_half = b_src(rb, kk);
+#pragma unroll
+      for (int n = 0; n < B_IT; ++n) b_half[n] = b_src(rb, kk, n);
       stage ^= 1;
     };
 
     // all k-tiles but the last; the first has no half refill to carry
     first_slices(nothing);
-    publish_next(!first_tile);
+    publish_next(prev_stored);
     final_slice(0);
     for (int kt = 1; kt + 1 < KT; ++kt) {
       first_slices(with_b_half);
@@ -1155,11 +1163,15 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     // fp16: requested a whole k-tile before it is needed; fp32 (twice the registers): in front
     // of the last slice
     typename Pack4<T>::type bias_raw[NB][4];
-    if constexpr (sizeof(T) == 2) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+    if constexpr (sizeof(T) == 2) {
+      if (wave_stores) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+    }
     __builtin_amdgcn_sched_barrier(0);
     first_slices(with_b_half);
     if (has_next) publish_next(false);
-    if constexpr (sizeof(T) == 4) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+    if constexpr (sizeof(T) == 4) {
+      if (wave_stores) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+    }
     __builtin_amdgcn_sched_barrier(0);
     slice(1, false, 0, 0, nothing);
     f4 bias_r[NB][4];
@@ -1172,7 +1184,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     stage ^= 1;
 
     // ---- epilogue: the next tile's first two k-tiles are landing meanwhile ----
-    {
+    if (wave_stores) {
       char* slab = smem + SLABS + wave * 4096;
       if constexpr (HALF_SLABS) {
         if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
@@ -1184,7 +1196,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     }
     if (!has_next) break;
     read_frags(stage, 0, 0);
-    first_tile = false;
+    prev_stored = wave_stores;
     vp = vp_next;
     m0 = m0_n;
     n0 = n0_n;
@@ -1256,8 +1268,15 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   auto a_src = [&](int m0, int k) __attribute__((always_inline)) {
     return (const char*)A + ((size_t)m0 * Kp * 2 + (size_t)k * ROWB);
   };
-  auto b_src = [&](int n0, int k) __attribute__((always_inline)) {
-    return (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+  // Source of load n (64-row block n) of the B tile at n0.  N is a multiple of 64, not
+  // necessarily of 256: in the last column tile a block that starts at or past row N loads
+  // block 0 again (the shift goes into the scalar source, the lane offsets stay); its products
+  // are never stored.
+  const size_t blk_bytes = (size_t)64 * Kp * 2;
+  auto b_src = [&](int n0, int k, int n) __attribute__((always_inline)) {
+    const int vb = (N - n0) >> 6;  // valid blocks of this tile (4 or more: all)
+    const char* p = (const char*)Bt + ((size_t)n0 * Kp * 2 + (size_t)k * ROWB);
+    return n < vb ? p : p - n * blk_bytes;
   };
   auto issue_a = [&](int stage, const char* src, int n) __attribute__((always_inline)) {
     lds_dma16_base(src, lane_off[n], wave_off + stage * STAGE + n * T_ * 16);
@@ -1267,11 +1286,10 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   };
   auto issue = [&](int stage, int m0, int n0, int k) __attribute__((always_inline)) {
     const char* a = a_src(m0, k);
-    const char* b = b_src(n0, k);
 #pragma unroll
     for (int n = 0; n < A_IT; ++n) issue_a(stage, a, n);
 #pragma unroll
-    for (int n = 0; n < B_IT; ++n) issue_b(stage, b, n);
+    for (int n = 0; n < B_IT; ++n) issue_b(stage, b_src(n0, k, n), n);
   };
   // Residual half h (rows 64 h .. 64 h + 63 of this wavefront's sub-tile) goes to the
   // wavefront's own 8 KB of `stage`: load q fetches 8 rows, lane l the 16-byte unit
@@ -1324,6 +1342,9 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     if (has_next) tile_origin(vp_next, m0_n, n0_n);
     const int64_t mw0 = (int64_t)m0 + wm * TM;
     const int nw0 = n0 + wn * TN;
+    // false: this wavefront's 64 columns lie past the edge -- it loads operands and keeps the
+    // barriers, and has no residual, bias or output of its own
+    const bool wave_stores = nw0 < N;
 
     f16v acc[NB][MB];
 #pragma unroll
@@ -1374,9 +1395,9 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
       wait_vmcnt<0>();
       barrier_lds();
     };
-    const char* b_half = nullptr;  // B half still to be issued into the other stage
+    const char* b_half[B_IT] = {};  // B half still to be issued into the other stage
     auto with_b_half = [&](int q) __attribute__((always_inline)) {
-      if (q & 1) issue_b(stage ^ 1, b_half, q / 2);
+      if (q & 1) issue_b(stage ^ 1, b_half[q / 2], q / 2);
     };
     // the final slice of a k-tile in front of the last but one: it takes the first fragments of
     // the published k-tile and starts the refill of this stage with the k-tile two ahead
@@ -1386,7 +1407,8 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
       slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
         if (q & 1) issue_a(stage, src, q / 2);
       });
-      b_half = b_src(n0, kt + 2);
+#pragma unroll
+      for (int n = 0; n < B_IT; ++n) b_half[n] = b_src(n0, kt + 2, n);
       stage ^= 1;
     };
 
@@ -1406,7 +1428,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     first_slices(with_b_half);
     publish_next();
     slice(1, true, stage ^ 1, 0, [&](int q) __attribute__((always_inline)) {
-      if (q & 1) issue_res_one(stage, res0, q / 2);
+      if ((q & 1) && wave_stores) issue_res_one(stage, res0, q / 2);
     });
     stage ^= 1;
 
@@ -1415,10 +1437,11 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     // the last slice and waited for behind it, before those loads are issued, so that no wait
     // the compiler places falls behind them.
     first_slices([&](int q) __attribute__((always_inline)) {
-      if (q & 1) issue_res_one(stage ^ 1, res0, 4 + q / 2);
+      if ((q & 1) && wave_stores) issue_res_one(stage ^ 1, res0, 4 + q / 2);
     });
     h4 bias_raw[NB][4];
-    load_bias<_Float16, NB>(ep, nw0, fhalf, bias_raw);  // all 8 loads in flight under the last slice
+    // all 8 loads in flight under the last slice
+    if (wave_stores) load_bias<_Float16, NB>(ep, nw0, fhalf, bias_raw);
     __builtin_amdgcn_sched_barrier(0);
     slice(1, false, 0, 0, nothing);
     f4 bias_r[NB][4];
@@ -1428,7 +1451,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
 #pragma unroll
       for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
     barrier_lds();  // every wavefront has read the last k-tile's fragments
-    {
+    if (wave_stores) {
       const char* res1 = res_src(m0, n0, 1);
 #pragma unroll
       for (int q = 0; q < 8; ++q) issue_res_one(stage, res1, q);
@@ -1436,7 +1459,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     stage ^= 1;  // now the stage of k-tile KT-2: the residual's first half, then the next tile's k-tile 0
 
     // ---- epilogue ----
-    {
+    if (wave_stores) {
       const char* res_lo = smem + stage * STAGE + wave * 8192;
       const char* res_hi = smem + (stage ^ 1) * STAGE + wave * 8192;
       char* slab = smem + SLABS + wave * 4096;
@@ -1452,12 +1475,17 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
       else
         store_wave_tile_rs<MB, NB, false>(acc, bias_r, ep, mw0, nw0, N, res_lo, res_hi, slab, lane,
                                           has_next, mid);
+    } else if (has_next) {
+      barrier_lds();  // the barrier and the refill of `mid`
+      issue(stage, m0_n, n0_n, 0);
     }
     if (!has_next) break;
     barrier_lds();  // nobody reads the second half any more
     issue(stage ^ 1, m0_n, n0_n, 1);
-    // the next tile's k-tile 0: younger are the 8 stores of row bands 2 and 3 and the 8 loads above
-    wait_vmcnt<16>();
+    // the next tile's k-tile 0: younger are the 8 stores of row bands 2 and 3 (of a wavefront
+    // that stores) and the 8 loads above
+    if (wave_stores) wait_vmcnt<16>();
+    else wait_vmcnt<8>();
     asm volatile("s_barrier" ::: "memory");
     read_frags(stage, 0, 0);
     vp = vp_next;
@@ -1525,7 +1553,7 @@ int launch_stream_res(const void* A, const void* Bt, int64_t M, int N, int Kp, c
   }
   const int num_cus = cu_count();
   if (num_cus < 0) return num_cus;
-  const int tiles_m = (int)(M / 256), tiles_n = N / 256;
+  const int tiles_m = (int)(M / 256), tiles_n = (N + 255) / 256;
   const int num_tiles = tiles_m * tiles_n;
   const int group_w = column_group(tiles_n, 256, Kp);
   const int grid = num_tiles < num_cus ? num_tiles : num_cus;
@@ -1542,11 +1570,11 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256) {
-    // Whole 256 x 256 tiles, at least two k-tiles, vector epilogue (16-byte stores for fp16), no
-    // dropout, no residual: the streaming kernel.  It has neither edge handling nor the
-    // generator; with a residual its epilogue loads queue behind the next tile's operand loads
-    // and it measured no faster.
-    if (M % 256 == 0 && N % 256 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
+    // Whole row tiles, N a multiple of 64 (the wavefronts of the last column tile whose 64
+    // columns lie past the edge store nothing), at least two k-tiles, vector epilogue (16-byte
+    // stores for fp16), no dropout, no residual: the streaming kernel.  It has neither row edge
+    // handling nor the generator.
+    if (M % 256 == 0 && N % 64 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
         (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr) {
       // Every persistent workgroup walks ceil(tiles / CUs) tiles, so a few tiles beyond a whole
       // number of rounds cost a full round.  Then the last rows leave the persistent launch --
@@ -1555,7 +1583,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
       // tiles; 597 of the 600 row tiles stay, 768 rows follow as 144 tiles of 128 x 128).
       const int cus = cu_count();
       if (cus < 0) return cus;
-      const int64_t tiles_m = M / 256, tiles_n = N / 256, tiles = tiles_m * tiles_n;
+      const int64_t tiles_m = M / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
       const int64_t rounds = tiles / cus, rem = tiles % cus;
       int64_t m_head = M;
       if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;
@@ -1571,13 +1599,14 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     if constexpr (sizeof(T) == 2 && !QKV) {
       if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&
           (((uintptr_t)ep.residual) & 15) == 0) {
-        if (M % 256 == 0 && N % 256 == 0 && Kp >= 192 && Kp <= (1 << 21)) {
-          // whole tiles everywhere and at least three k-tiles: the streaming kernel, with the same cut as above -- the row
-          // tiles that fill whole rounds of the persistent workgroups stay, the rest (headline
-          // N = 768: 1800 tiles = 7 rounds + 8; 597 of 600 row tiles stay) go to the small tiles
+        if (M % 256 == 0 && N % 64 == 0 && Kp >= 192 && Kp <= (1 << 21)) {
+          // whole row tiles, N a multiple of 64 and at least three k-tiles: the streaming
+          // kernel, with the same cut as above -- the row tiles that fill whole rounds of the
+          // persistent workgroups stay, the rest (headline N = 768: 1800 tiles = 7 rounds + 8;
+          // 597 of 600 row tiles stay) go to the small tiles
           const int cus = cu_count();
           if (cus < 0) return cus;
-          const int64_t tiles_m = M / 256, tiles_n = N / 256, tiles = tiles_m * tiles_n;
+          const int64_t tiles_m = M / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
           const int64_t rounds = tiles / cus, rem = tiles % cus;
           int64_t m_head = M;
           if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;

@@ -92,6 +92,10 @@ def test_headline_gemm_every_element(K, gpu_device, name, Kd, N, gelu, use_res, 
     (66560, 1024, 256, False, True, True),    # 1040 tiles = 4 rounds + 16: head + small-tile tail,
                                               # output written over the residual
     (4096, 768, 3072, False, True, False),    # 48 tiles: one each, nothing to refill
+    (16384, 1600, 320, False, True, False),   # N = 6 x 256 + 64: three of four wavefront columns
+                                              # of the last column tile lie past the edge
+    (8192, 320, 256, True, True, True),       # two column tiles, the second 64 wide; in place
+    (2048, 448, 192, False, True, False),     # 8 + 8 tiles, three k-tiles, last tile 192 wide
 ])
 def test_residual_gemm_streaming_every_element(K, gpu_device, M, N, Kd, gelu, bias, in_place):
     """fp16 GEMM + residual on whole 256 x 256 tiles (the persistent kernel that carries the
@@ -118,6 +122,37 @@ def test_residual_gemm_streaming_every_element(K, gpu_device, M, N, Kd, gelu, bi
         z = torch.full((M, N), float("nan"), device=gpu_device, dtype=torch.float16)
         K._linear(x, K.pack_weight(w), b, res, z, gelu, 0.0, K._lib.GPTMI_W_PACKED, "residual")
     assert_all_close_f16(z, want, "residual streaming")
+
+
+@pytest.mark.parametrize("M,N,Kd,gelu,dtype", [
+    (8192, 1600, 256, True, torch.float16),   # 6 whole column tiles + 64 columns
+    (4096, 4800, 128, False, torch.float16),  # 18 whole column tiles + 192 columns
+    (2048, 448, 192, True, torch.float32),    # fp32 output: the other epilogue of the kernel
+    (2048, 320, 128, False, torch.float16),   # two k-tiles, second column tile 64 wide
+])
+def test_gemm_streaming_ragged_columns_every_element(K, gpu_device, M, N, Kd, gelu, dtype):
+    """GEMM + bias (+ GELU) without residual where N is a multiple of 64 and not of 256: the
+    persistent kernel's last column tile has wavefronts whose columns lie past the edge (they
+    load operands, keep the barriers and store nothing).  Every element against the fp32 torch
+    product of the fp16-rounded operands; the output buffer is NaN-poisoned and followed by a
+    guard row that must stay untouched."""
+    g = torch.Generator(device=gpu_device).manual_seed(N + Kd)
+    x = torch.randn((M, Kd), generator=g, device=gpu_device).to(dtype)
+    w = (torch.randn((Kd, N), generator=g, device=gpu_device) / Kd ** 0.5).to(dtype)
+    b = (0.1 * torch.randn(N, generator=g, device=gpu_device)).to(dtype)
+    want = x.half().float() @ w.half().float() + b.float()
+    if gelu:
+        want = gelu_tanh(want)
+    buf = torch.full((M + 1, N), float("nan"), device=gpu_device, dtype=dtype)
+    z = buf[:M]
+    print(f"ragged columns: M={M} N={N} K={Kd} gelu={gelu} {dtype}", flush=True)
+    K._linear(x, K.pack_weight(w), b, None, z, gelu, 0.0, K._lib.GPTMI_W_PACKED, "ragged")
+    assert torch.isnan(buf[M]).all(), "wrote past the last row"
+    if dtype == torch.float16:
+        assert_all_close_f16(z, want, "ragged columns")
+    else:
+        assert torch.isfinite(z).all()
+        torch.testing.assert_close(z, want, rtol=2e-4, atol=2e-4)
 
 
 def test_headline_qkv_every_element(K, gpu_device):
