@@ -1562,6 +1562,23 @@ int launch_stream_res(const void* A, const void* Bt, int64_t M, int N, int Kp, c
   return 0;
 }
 
+// Problems too small for the 256 x 256 tiles (and the last rows of the persistent launches): 4
+// wavefronts on 128 x 128 tiles, K step 32, 4-stage ring -- unless that leaves most CUs without
+// a workgroup; then smaller tiles with a K step of 64, so that the few k-tiles a workgroup walks
+// (each a barrier and an LDS round trip) are as few as possible.  Last 768 rows of the headline
+// GEMMs, one box: N = 768, K = 3072: 40 -> 19 us; N = K = 768: 15 -> 8; N = 2304: 15 -> 10;
+// N = 3072: 14.6 -> 12.5.
+template <typename T, bool QKV>
+int launch_small(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+                 hipStream_t st) {
+  const int cus = cu_count();
+  if (cus < 0) return cus;
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles128 * 4 <= cus) return launch_cfg<64, 64, 2, 1, 64, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  if (tiles128 <= cus) return launch_cfg<64, 128, 2, 2, 64, 3, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+}
+
 template <typename T, bool QKV>
 int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
                  hipStream_t st) {
@@ -1580,7 +1597,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
       // number of rounds cost a full round.  Then the last rows leave the persistent launch --
       // as many row tiles stay as fill whole rounds -- and go to the small-tile kernel, whose
       // many short workgroups spread over all CUs (headline ffn1: 7200 tiles = 28 rounds + 32
-      // tiles; 597 of the 600 row tiles stay, 768 rows follow as 144 tiles of 128 x 128).
+      // tiles; 597 of the 600 row tiles stay, 768 rows follow as 288 tiles of 64 x 128).
       const int cus = cu_count();
       if (cus < 0) return cus;
       const int64_t tiles_m = M / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
@@ -1592,7 +1609,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
       EpiDev tail = ep;
       if (QKV) tail.m_off = ep.m_off + (int)m_head;
       else tail.out = (T*)ep.out + m_head * N;
-      return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>((const _Float16*)A + m_head * Kp, Bt,
+      return launch_small<T, QKV>((const _Float16*)A + m_head * Kp, Bt,
                                                           M - m_head, N, Kp, tail, st);
     }
     // fp16 with a residual, no dropout: whole tiles fetch the residual through LDS
@@ -1615,7 +1632,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
           EpiDev tail = ep;
           tail.out = (T*)ep.out + m_head * N;
           tail.residual = (const T*)ep.residual + m_head * N;
-          return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>((const _Float16*)A + m_head * Kp, Bt,
+          return launch_small<T, QKV>((const _Float16*)A + m_head * Kp, Bt,
                                                               M - m_head, N, Kp, tail, st);
         }
         return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV, true>(A, Bt, M, N, Kp, ep, st);
@@ -1623,7 +1640,7 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     }
     return launch_cfg<256, 256, 2, 4, 64, 2, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
   }
-  return launch_cfg<128, 128, 2, 2, 32, 4, 2, T, QKV>(A, Bt, M, N, Kp, ep, st);
+  return launch_small<T, QKV>(A, Bt, M, N, Kp, ep, st);
 }
 
 }  // namespace
