@@ -387,12 +387,6 @@ int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int
     set_error("flash_attn: invalid argument");
     return GPTMI_ERR_INVALID;
   }
-  if (Lq != Lk) {
-    set_error("flash_attn: Lq=%lld != Lk=%lld is not supported (the causal mask is "
-              "top-left aligned and padded keys rely on it)",
-              (long long)Lq, (long long)Lk);
-    return GPTMI_ERR_UNSUPPORTED;
-  }
   if (!dropout_ok(p)) {
     set_error("flash_attn: dropout probability %g outside [0, 1)", (double)p);
     return GPTMI_ERR_INVALID;
@@ -402,7 +396,7 @@ int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int
     set_error("flash_attn: q, k, v and out must be 16-byte aligned");
     return GPTMI_ERR_INVALID;
   }
-  int rc = launch_flash_attn(q, k, v, out, B, N, Lq, (int)d, scale, Dropout{p, seed},
+  int rc = launch_flash_attn(q, k, v, out, B, N, Lq, Lk, (int)d, scale, Dropout{p, seed},
                              olayout == GPTMI_O_BLND,
                              dtype == GPTMI_F16, (hipStream_t)stream);
   if (rc) return rc;

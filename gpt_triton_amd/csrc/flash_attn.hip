@@ -73,7 +73,10 @@ __device__ __forceinline__ h8 zero_h8() {
 template <int D, typename T, bool BLND, bool DROP>
 __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-    T* __restrict__ O, int heads, int L, float scale, DropoutArgs drop) {
+    T* __restrict__ O, int heads, int L, int Lk, float scale, DropoutArgs drop) {
+  // L = query rows, Lk = key rows of every (batch, head).  The mask is "key <= query" alone and
+  // key rows at or past Lk count as zero rows, as in the reference (kernels.py:421-436): with
+  // L > Lk the queries at or past Lk also see the zero rows that fill up the last key tile.
   constexpr int CH = D / 8;             // 16-byte chunks per row
   constexpr int KS = D / 16;            // MFMA k-steps over the head dim
   constexpr int DB = D / 32;            // 32-row blocks of O^T
@@ -89,10 +92,10 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   // heavy (late) query blocks first so the tail of the grid is light
   const int qb = q_blocks - 1 - (int)blockIdx.y;
   const int q0 = qb * BQ;
-  const int64_t base = (int64_t)bh * L * D;
+  const int64_t base = (int64_t)bh * L * D, kv_base = (int64_t)bh * Lk * D;
   const T* Qp = Q + base;
-  const T* Kp = K + base;
-  const T* Vp = V + base;
+  const T* Kp = K + kv_base;
+  const T* Vp = V + kv_base;
 
   const int ql = lane & 31, g = lane >> 5;
   const int qw0 = q0 + wave * 32;    // first query of this wavefront
@@ -107,14 +110,15 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
 
   int last_q = q0 + BQ - 1;
   if (last_q > L - 1) last_q = L - 1;
-  const int nt = last_q / BKEY + 1;  // key tiles 0..nt-1 touch this query block
+  // key tiles 0..nt-1 touch this query block: up to the diagonal, and no further than the keys go
+  const int nt = min(last_q / BKEY + 1, (Lk + BKEY - 1) / BKEY);
 
   // ---- staging: each thread moves NLD 16-byte chunks per tile --------------
   // waves 0-1 (role K): chunk s = i*128 + st -> key s / CH, chunk s % CH
   // waves 2-3 (role V): unit  s = (i/4)*128 + st -> key group s & 15 (4 keys),
   //                     chunk s >> 4; register i holds key 4*group + i%4.
-  // Rows past the end of the sequence are clamped to the last row: their keys
-  // are masked (P = 0 exactly) and the values stay finite.
+  // Rows at or past Lk are zero rows: invisible to every valid query when L <= Lk (their keys
+  // are masked, P = 0 exactly), visible padding when L > Lk.
   constexpr int NLD = K_LD;
   static_assert(K_LD == 4 * V_UNITS, "K and V staging must move the same chunk count");
   const int st = tid & 127;
@@ -142,9 +146,8 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     const int k0 = t * BKEY;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      int row = k0 + srow[i];
-      row = row < L ? row : L - 1;
-      dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
+      const int row = k0 + srow[i];
+      dst[i] = row < Lk ? Ld8<T>::load(sp + (int64_t)row * D + scol[i]) : zero_h8();
     }
   };
 
@@ -266,13 +269,13 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
       den = den * mult + psum;
       if constexpr (DROP) {
         // dropout of P after the denominator has summed it, before the fp16 rounding;
-        // offset = query * L + key, the same for every batch and head (kernels.py:457-460)
+        // offset = query * Lk + key, the same for every batch and head (kernels.py:457-460)
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int rg = 0; rg < 4; ++rg) {
             const unsigned key0 = (unsigned)(k0 + kb * 32 + 8 * rg + 4 * g);
-            const unsigned base_off = (unsigned)q * (unsigned)L + key0;
+            const unsigned base_off = (unsigned)q * (unsigned)Lk + key0;
             unsigned off[4] = {base_off, base_off + 1u, base_off + 2u, base_off + 3u};
             float pv[4] = {s[kb][4 * rg], s[kb][4 * rg + 1], s[kb][4 * rg + 2], s[kb][4 * rg + 3]};
             dropout_apply<4>(drop, off, pv);
@@ -967,7 +970,7 @@ int launch_resident(const void* q, const void* k, const void* v, void* out, int6
 
 template <int D, typename T, bool BLND, bool DROP>
 int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
-                 int L, float scale, DropoutArgs drop, hipStream_t st) {
+                 int L, int Lk, float scale, DropoutArgs drop, hipStream_t st) {
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
   constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V^T tile
   auto kern = flash_attn_kernel<D, T, BLND, DROP>;
@@ -982,7 +985,7 @@ int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t
   }
   attr_done = true;
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
-                     (T*)out, heads, L, scale, drop);
+                     (T*)out, heads, L, Lk, scale, drop);
   return 0;
 }
 
@@ -1028,12 +1031,15 @@ int launch_stream_attn(const void* q, const void* k, const void* v, void* out, i
 
 template <int D, typename T>
 int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
-             int heads, int L, float scale, Dropout drop, bool blnd, hipStream_t st) {
+             int heads, int L, int Lk, float scale, Dropout drop, bool blnd, hipStream_t st) {
   const DropoutArgs da = {drop.p, (unsigned)drop.seed, (unsigned)(drop.seed >> 32)};
   if (drop.p > 0.f) {  // training-mode path: the tiled kernel carries the generator
-    return blnd ? launch_tiled<D, T, true, true>(q, k, v, out, BN, heads, L, scale, da, st)
-                : launch_tiled<D, T, false, true>(q, k, v, out, BN, heads, L, scale, da, st);
+    return blnd ? launch_tiled<D, T, true, true>(q, k, v, out, BN, heads, L, Lk, scale, da, st)
+                : launch_tiled<D, T, false, true>(q, k, v, out, BN, heads, L, Lk, scale, da, st);
   }
+  if (L != Lk)  // query and key sequences of different lengths: the tiled kernel knows both
+    return blnd ? launch_tiled<D, T, true, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st)
+                : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st);
   if constexpr (D == 64 && sizeof(T) == 2) {
     // fp16, head size 64, two (batch, head) pairs fit the LDS, enough pairs to keep every
     // persistent workgroup busy for a while: the streaming kernel
@@ -1045,17 +1051,17 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
     return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
                 : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
   }
-  return blnd ? launch_tiled<D, T, true, false>(q, k, v, out, BN, heads, L, scale, da, st)
-              : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, scale, da, st);
+  return blnd ? launch_tiled<D, T, true, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st)
+              : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st);
 }
 
 template <typename T>
 int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
-             int heads, int L, int d, float scale, Dropout drop, bool blnd, hipStream_t st) {
+             int heads, int L, int Lk, int d, float scale, Dropout drop, bool blnd, hipStream_t st) {
   switch (d) {
-    case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
-    case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
-    case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, scale, drop, blnd, st);
+    case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
+    case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
+    case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
     default:
       set_error("flash_attn: head size %d not built (64, 128 and 256 are)", d);
       return -2;
@@ -1065,16 +1071,18 @@ int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
 }  // namespace
 
 int launch_flash_attn(const void* q, const void* k, const void* v, void* out, int64_t B,
-                      int64_t N, int64_t L, int d, float scale, Dropout drop, bool out_blnd,
-                      bool f16, hipStream_t st) {
+                      int64_t N, int64_t L, int64_t Lk, int d, float scale, Dropout drop,
+                      bool out_blnd, bool f16, hipStream_t st) {
   const int64_t BN = B * N;
-  if (BN > 0x7fffffffll || L > (1 << 24)) {
-    set_error("flash_attn: B*N=%lld or L=%lld beyond the grid limits", (long long)BN,
-              (long long)L);
+  if (BN > 0x7fffffffll || L > (1 << 24) || Lk > (1 << 24)) {
+    set_error("flash_attn: B*N=%lld, Lq=%lld or Lk=%lld beyond the grid limits", (long long)BN,
+              (long long)L, (long long)Lk);
     return -2;
   }
-  return f16 ? launch_t<_Float16>(q, k, v, out, BN, (int)N, (int)L, d, scale, drop, out_blnd, st)
-             : launch_t<float>(q, k, v, out, BN, (int)N, (int)L, d, scale, drop, out_blnd, st);
+  return f16 ? launch_t<_Float16>(q, k, v, out, BN, (int)N, (int)L, (int)Lk, d, scale, drop,
+                                  out_blnd, st)
+             : launch_t<float>(q, k, v, out, BN, (int)N, (int)L, (int)Lk, d, scale, drop, out_blnd,
+                               st);
 }
 
 }  // namespace gptmi

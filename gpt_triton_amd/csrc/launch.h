@@ -49,8 +49,9 @@ struct GemmEpilogue {
 int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
                 const GemmEpilogue& ep, hipStream_t st);
 
+// q, out: L rows per (batch, head); k, v: Lk rows.
 int launch_flash_attn(const void* q, const void* k, const void* v, void* out,
-                      int64_t B, int64_t N, int64_t L, int d, float scale, Dropout drop,
-                      bool out_blnd, bool f16, hipStream_t st);
+                      int64_t B, int64_t N, int64_t L, int64_t Lk, int d, float scale,
+                      Dropout drop, bool out_blnd, bool f16, hipStream_t st);
 
 }  // namespace gptmi

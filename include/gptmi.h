@@ -223,7 +223,12 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
  *
  * Replaces flash_attention_v1(q, k, v, dropout_prob) -> kernels.py:477-525 and
  * flash_attention_v1_kernel -> kernels.py:375-474.
- *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64, 128 or 256    Lq == Lk
+ *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64, 128 or 256
+ * Lq != Lk behaves as in the reference (kernels.py:421-436): the mask is "key <= query" from the
+ * top left, nothing else, and the last 64-key tile is filled up with zero rows.  So with Lq < Lk
+ * the keys past the last query play no part, and with Lq > Lk a query at or past Lk attends to all
+ * Lk keys AND to the zero rows Lk .. min(query, round_up(Lk, 64) - 1) (score 0, value 0), which
+ * only add to its denominator.
  *   out: [B][N][Lq][d] (GPTMI_O_BNLD) or [B][Lq][N][d] (GPTMI_O_BLND)
  * Dropout (0 < p < 1; 0 = none) hits P after the denominator has summed it and before its
  * fp16 rounding (kernels.py:457-466): keep where rand(seed, (uint32)(lq*Lk + lk)) > p,

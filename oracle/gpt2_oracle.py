@@ -209,7 +209,7 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
 
 
 def flash_attention_v1(q, k, v, block=BLOCK_L, dropout_prob=0.0, seed=SEED):
-    """kernels.py:408-474, Lq == Lk.  Dropout (p > 0 only) hits P after the denominator has
+    """kernels.py:408-474.  Dropout (p > 0 only) hits P after the denominator has
     summed it and before the fp16 rounding, offset = lq * Lk + lk for every batch and head
     (kernels.py:457-460).
 
@@ -217,20 +217,30 @@ def flash_attention_v1(q, k, v, block=BLOCK_L, dropout_prob=0.0, seed=SEED):
     fp32; causal mask; running max m; P = exp(S - m_new); den = den * exp(m - m_new) +
     sum(P) with P unrounded; acc = acc * exp(m - m_new) + fp16(P) . v16 in fp32;
     out = acc / den.
+
+    Lq != Lk (q [B, N, Lq, D]; k, v [B, N, Lk, D]) as the reference has it: the mask is
+    `query >= key` alone (kernels.py:436) and the last key tile is filled up with zero rows
+    (kernels.py:421-424, 462), so a query at or past Lk also attends to that padding (score 0,
+    value 0); keys past the last query are never visible.  With Lq == Lk no valid query sees a
+    padding row, and the tile may end at Lk.
     """
     out_dtype = q.dtype
-    B, N, L, D = q.shape
-    assert k.shape == q.shape and v.shape == q.shape
+    B, N, Lq, D = q.shape
+    Lk = k.shape[2]
+    assert k.shape == (B, N, Lk, D) and v.shape == k.shape
     scale = F32(1.0 / math.sqrt(D))  # a Python float in the reference, fp32 on the device
-    q16 = round_to_f16(q).reshape(B * N, L, D)
-    k16 = round_to_f16(k).reshape(B * N, L, D)
-    v16 = round_to_f16(v).reshape(B * N, L, D)
-    acc = np.zeros((B * N, L, D), dtype=F32)
-    mrun = np.full((B * N, L, 1), -np.inf, dtype=F32)
-    den = np.zeros((B * N, L, 1), dtype=F32)
-    rows = np.arange(L)[:, None]
-    for k0 in range(0, L, block):
-        k1 = min(k0 + block, L)
+    Lkp = Lk if Lq <= Lk else -(-Lk // block) * block  # zero rows that a query can see
+    q16 = round_to_f16(q).reshape(B * N, Lq, D)
+    k16 = np.zeros((B * N, Lkp, D), dtype=F32)
+    v16 = np.zeros((B * N, Lkp, D), dtype=F32)
+    k16[:, :Lk] = round_to_f16(k).reshape(B * N, Lk, D)
+    v16[:, :Lk] = round_to_f16(v).reshape(B * N, Lk, D)
+    acc = np.zeros((B * N, Lq, D), dtype=F32)
+    mrun = np.full((B * N, Lq, 1), -np.inf, dtype=F32)
+    den = np.zeros((B * N, Lq, 1), dtype=F32)
+    rows = np.arange(Lq)[:, None]
+    for k0 in range(0, Lkp, block):
+        k1 = min(k0 + block, Lkp)
         cols = np.arange(k0, k1)[None, :]
         s = np.matmul(q16, k16[:, k0:k1].transpose(0, 2, 1), dtype=F32) * scale
         s = np.where(rows >= cols, s, F32(-np.inf))
@@ -241,11 +251,11 @@ def flash_attention_v1(q, k, v, block=BLOCK_L, dropout_prob=0.0, seed=SEED):
             mult = np.exp(mrun - mnew)
         den = den * mult + p.sum(axis=2, dtype=F32, keepdims=True)
         if dropout_prob > 0.0:
-            p = dropout(p, dropout_prob, seed, (rows * L + cols)[None])
+            p = dropout(p, dropout_prob, seed, (rows * Lk + cols)[None])
         acc = acc * mult + np.matmul(round_to_f16(p), v16[:, k0:k1], dtype=F32)
         mrun = mnew
     out = acc / den
-    return out.astype(out_dtype).reshape(B, N, L, D)
+    return out.astype(out_dtype).reshape(B, N, Lq, D)
 
 
 def softmax_rows(x):

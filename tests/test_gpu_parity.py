@@ -477,6 +477,36 @@ def test_flash_attention_small_heads(K, gpu_device, dtype, D):
     assert np.array_equal(host(zm), host(z))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_flash_attention_unequal_lengths_reference_golden_vectors(K, gpu_device, dtype):
+    """Lq != Lk against outputs of the reference's own kernel (Triton CPU interpreter,
+    tests/golden/make_flash_lqlk_vectors.py): keys past the last query play no part; queries at
+    or past Lk also see the zero rows that fill up the last key tile (kernels.py:421-436)."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "flash_attention_v1_lq_lk.npz"))
+    for n in ("short_q", "long_q", "long_q_whole_tile", "long_q_d128"):
+        q, k, v = (z[f"{n}_{t}"].astype(NP[dtype]) for t in "qkv")
+        got = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+        assert got.shape == q.shape
+        check_attention(host(got), z[f"{n}_out"], v, dtype, f"golden {n}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("Lq,Lk", [(1, 5), (5, 1), (64, 65), (65, 64), (300, 129), (129, 300),
+                                   (700, 200), (200, 700)])
+def test_flash_attention_unequal_lengths(K, gpu_device, dtype, Lq, Lk):
+    r = np.random.default_rng(Lq * 1000 + Lk)
+    q = r.standard_normal((2, 3, Lq, 64)).astype(NP[dtype])
+    k, v = (r.standard_normal((2, 3, Lk, 64)).astype(NP[dtype]) for _ in range(2))
+    want = O.flash_attention_v1(q, k, v)
+    for merged in (False, True):
+        z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                                 merged_heads_layout=merged)
+        assert z.shape == (2, 3, Lq, 64)
+        check_attention(host(z), want, v, dtype, f"attention Lq={Lq} Lk={Lk}")
+
+
 def test_flash_attention_xl_sequence(K, gpu_device):
     """Benchmark configuration 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
     K/V do not fit the resident variant)."""
@@ -836,6 +866,18 @@ def test_dropout_attention(K, gpu_device, dtype, B, N, L, D):
     zm = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
                               dropout_prob=0.2, merged_heads_layout=True)
     assert np.array_equal(host(zm), z)
+
+
+@pytest.mark.parametrize("Lq,Lk", [(100, 180), (180, 100)])
+def test_dropout_attention_unequal_lengths(K, gpu_device, Lq, Lk):
+    """The generator's offset is query * Lk + key (kernels.py:458): Lk, not Lq, is the pitch."""
+    r = np.random.default_rng(33)
+    q = r.standard_normal((1, 2, Lq, 64)).astype(np.float16)
+    k, v = (r.standard_normal((1, 2, Lk, 64)).astype(np.float16) for _ in range(2))
+    z = host(K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                                  dropout_prob=0.2))
+    want = O.flash_attention_v1(q, k, v, dropout_prob=0.2)
+    check_attention(z, want, v.astype(np.float32) / 0.8, torch.float16, "attention dropout")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])

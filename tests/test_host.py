@@ -56,8 +56,8 @@ def test_invalid_arguments_are_rejected_before_any_launch(lib):
     assert lib.gptmi_embed(fake, fake, fake, fake, 1, 4, 4, 4, 8, 1.0, 0, 1, None) == -1  # p >= 1
     assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 8, 64, 0.125, -0.1, 0, 0, 1,
                                 None) == -1                                             # p < 0
-    assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 9, 64, 0.125, 0.0, 0, 0, 1,
-                                None) == -2                                             # Lq != Lk
+    assert lib.gptmi_flash_attn(fake, fake, fake, fake, 1, 1, 8, 9, 48, 0.125, 0.0, 0, 0, 1,
+                                None) == -2                                             # head size
     # output rows wider than the epilogues' 32-bit lane offsets can address: refused, not wrapped
     wide = (1 << 26) + 8
     assert lib.gptmi_linear(fake, fake, None, None, fake, 4, wide, 64, 0, 0.0, 0, 2, None, 0, 1,

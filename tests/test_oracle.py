@@ -280,6 +280,57 @@ def test_attention_vs_reference_golden_vectors():
         assert np.abs(other.astype(np.float64) - want).max() > 20 * diff.max()
 
 
+def test_attention_unequal_lengths_vs_reference_golden_vectors():
+    """tests/golden/flash_attention_v1_lq_lk.npz: the reference's flash_attention_v1 with
+    Lq != Lk (Triton CPU interpreter, tests/golden/make_flash_lqlk_vectors.py).  The vectors pin
+    the two things only the reference's code decides: keys past the last query are invisible
+    (Lq < Lk), and the zero rows that fill up the last key tile are visible to the queries at or
+    past Lk (Lq > Lk)."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "flash_attention_v1_lq_lk.npz"))
+    for n in ("short_q", "long_q", "long_q_whole_tile", "long_q_d128"):
+        q, k, v = (z[f"{n}_{t}"].astype(np.float32) for t in "qkv")
+        want = z[f"{n}_out"]
+        got = O.flash_attention_v1(q, k, v)
+        diff = np.abs(got.astype(np.float64) - want)
+        assert diff.max() <= 2e-7 * np.abs(want).max(), n
+        assert (diff == 0).mean() > 0.95, n
+    # the vectors against the textbook, written out independently of the oracle: softmax over the
+    # visible keys, where a padding row counts as a key with score 0 and value 0
+    for n, pad_to in (("short_q", None), ("long_q", 128), ("long_q_whole_tile", 64),
+                      ("long_q_d128", 64)):
+        q, k, v = (z[f"{n}_{t}"].astype(np.float64) for t in "qkv")
+        want = z[f"{n}_out"]
+        Lq, Lk, D = q.shape[2], k.shape[2], q.shape[3]
+        for bn in range(q.shape[1]):
+            for i in (0, Lq // 3, Lq - 1):
+                vis = min(i + 1, Lk)
+                s = (k[0, bn, :vis] @ q[0, bn, i]) / np.sqrt(D)
+                zeros = 0 if pad_to is None else max(0, min(i + 1, pad_to) - Lk)
+                s_all = np.concatenate([s, np.zeros(zeros)])
+                w = np.exp(s_all - s_all.max())
+                out = (w[:vis, None] * v[0, bn, :vis]).sum(0) / w.sum()
+                assert np.abs(out - want[0, bn, i]).max() <= 2.0**-10 * np.abs(v).max(), (n, i)
+    # a plausible mistake -- masking the padding rows by Lk -- is told apart by the vectors
+    q, k, v = (z[f"long_q_{t}"].astype(np.float64) for t in "qkv")
+    i = 149
+    s = (k[0, 0] @ q[0, 0, i]) / 8.0
+    w = np.exp(s - s.max())
+    no_pad = (w[:, None] * v[0, 0]).sum(0) / w.sum()
+    assert np.abs(no_pad - z["long_q_out"][0, 0, i]).max() > 1e-2
+
+
+def test_attention_shorter_queries_equal_truncated_keys():
+    # Lq < Lk: exactly the attention over the first Lq keys (later tiles add exact zeros)
+    r = rng(41)
+    q = r.standard_normal((1, 2, 90, 64)).astype(np.float32)
+    k, v = (r.standard_normal((1, 2, 200, 64)).astype(np.float32) for _ in range(2))
+    a = O.flash_attention_v1(q, k, v)
+    b = O.flash_attention_v1(q, k[:, :, :90], v[:, :, :90])
+    assert np.array_equal(a, b)
+
+
 # ----------------------------------------------------------------------------- softmax
 def test_softmax_vs_torch():
     r = rng(37)
