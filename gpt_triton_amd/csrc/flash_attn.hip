@@ -70,13 +70,16 @@ __device__ __forceinline__ h8 zero_h8() {
 // D = head size.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
 // position c ^ (r&7)) and V^T tile [D][64] (8-byte unit u of row d at position
 // u ^ ((d>>1)&15)).
-template <int D, typename T, bool BLND, bool DROP>
+template <int D, typename T, bool BLND, bool DROP, bool UNEQ>
 __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-    T* __restrict__ O, int heads, int L, int Lk, float scale, DropoutArgs drop) {
-  // L = query rows, Lk = key rows of every (batch, head).  The mask is "key <= query" alone and
-  // key rows at or past Lk count as zero rows, as in the reference (kernels.py:421-436): with
-  // L > Lk the queries at or past Lk also see the zero rows that fill up the last key tile.
+    T* __restrict__ O, int heads, int L, int Lk_arg, float scale, DropoutArgs drop) {
+  // L = query rows, Lk = key rows of every (batch, head); UNEQ = they may differ.  The mask is
+  // "key <= query" alone and key rows at or past Lk count as zero rows, as in the reference
+  // (kernels.py:421-436): with L > Lk the queries at or past Lk also see the zero rows that fill
+  // up the last key tile.  With L == Lk no valid query sees such a row, and the staging loads
+  // read the last row again instead (no select per load).
+  const int Lk = UNEQ ? Lk_arg : L;
   constexpr int CH = D / 8;             // 16-byte chunks per row
   constexpr int KS = D / 16;            // MFMA k-steps over the head dim
   constexpr int DB = D / 32;            // 32-row blocks of O^T
@@ -111,14 +114,14 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   int last_q = q0 + BQ - 1;
   if (last_q > L - 1) last_q = L - 1;
   // key tiles 0..nt-1 touch this query block: up to the diagonal, and no further than the keys go
-  const int nt = min(last_q / BKEY + 1, (Lk + BKEY - 1) / BKEY);
+  const int nt = UNEQ ? min(last_q / BKEY + 1, (Lk + BKEY - 1) / BKEY) : last_q / BKEY + 1;
 
   // ---- staging: each thread moves NLD 16-byte chunks per tile --------------
   // waves 0-1 (role K): chunk s = i*128 + st -> key s / CH, chunk s % CH
   // waves 2-3 (role V): unit  s = (i/4)*128 + st -> key group s & 15 (4 keys),
   //                     chunk s >> 4; register i holds key 4*group + i%4.
-  // Rows at or past Lk are zero rows: invisible to every valid query when L <= Lk (their keys
-  // are masked, P = 0 exactly), visible padding when L > Lk.
+  // Rows at or past Lk: zero rows if the lengths may differ (visible padding when L > Lk);
+  // otherwise the last row again -- the keys are masked (P = 0 exactly), the values finite.
   constexpr int NLD = K_LD;
   static_assert(K_LD == 4 * V_UNITS, "K and V staging must move the same chunk count");
   const int st = tid & 127;
@@ -146,8 +149,13 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     const int k0 = t * BKEY;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int row = k0 + srow[i];
-      dst[i] = row < Lk ? Ld8<T>::load(sp + (int64_t)row * D + scol[i]) : zero_h8();
+      int row = k0 + srow[i];
+      if constexpr (UNEQ) {
+        dst[i] = row < Lk ? Ld8<T>::load(sp + (int64_t)row * D + scol[i]) : zero_h8();
+      } else {
+        row = row < L ? row : L - 1;
+        dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
+      }
     }
   };
 
@@ -968,12 +976,12 @@ int launch_resident(const void* q, const void* k, const void* v, void* out, int6
   return 0;
 }
 
-template <int D, typename T, bool BLND, bool DROP>
-int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
-                 int L, int Lk, float scale, DropoutArgs drop, hipStream_t st) {
+template <int D, typename T, bool BLND, bool DROP, bool UNEQ>
+int launch_tiled_as(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                    int L, int Lk, float scale, DropoutArgs drop, hipStream_t st) {
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
   constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V^T tile
-  auto kern = flash_attn_kernel<D, T, BLND, DROP>;
+  auto kern = flash_attn_kernel<D, T, BLND, DROP, UNEQ>;
   static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done && lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -987,6 +995,16 @@ int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const T*)q, (const T*)k, (const T*)v,
                      (T*)out, heads, L, Lk, scale, drop);
   return 0;
+}
+
+// L query rows, Lk key rows per (batch, head); equal lengths take the variant without the
+// zero-row selects.
+template <int D, typename T, bool BLND, bool DROP>
+int launch_tiled(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                 int L, int Lk, float scale, DropoutArgs drop, hipStream_t st) {
+  if (L != Lk)
+    return launch_tiled_as<D, T, BLND, DROP, true>(q, k, v, out, BN, heads, L, Lk, scale, drop, st);
+  return launch_tiled_as<D, T, BLND, DROP, false>(q, k, v, out, BN, heads, L, Lk, scale, drop, st);
 }
 
 // CUs of the current device, or a negative error code.
