@@ -44,10 +44,10 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
 }
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
-# HBM-side bytes of one ffn1 launch from rocprofv3 --pmc FETCH_SIZE (1001.8 MB after scaling by
-# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.8 MB); the counters cannot be read
+# HBM-side bytes of one ffn1 call from rocprofv3 --pmc FETCH_SIZE (992.4 MB after scaling by
+# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.9 MB); the counters cannot be read
 # from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
-FFN1_TRAFFIC_BYTES = 1.946e9
+FFN1_TRAFFIC_BYTES = 1.936e9
 
 
 def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
