@@ -892,13 +892,17 @@ __global__ __launch_bounds__(512, 2) void flash_attn_stream_kernel(
   if (c0 >= 0) load_q(bh, c0, q_heavy_next);
   if (c1 >= 0) load_q(bh, c1, q_light);
   int buf = 0;
+  bool stored = false;  // this wavefront's heavy chunk stored its 4 x 16 bytes right before
   while (true) {
     const int bh_next = bh + (int)gridDim.x;
     const bool has_next = bh_next < num_bh;
-    // everything this wavefront requested has landed (the pair's K / V units and queries, and
-    // the previous pair's stores); behind the barrier that holds for every wavefront, and
-    // nobody reads the other buffer any more
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // Everything this wavefront LOADED has landed (the pair's K / V units and queries); behind the
+    // barrier that holds for every wavefront, and nobody reads the other buffer any more.  Loads
+    // and stores retire in issue order, and the only operations younger than the last load are the
+    // four output stores of the heavy chunk: waiting until four are outstanding leaves exactly
+    // those in flight instead of waiting ~2 us for their acknowledgements once per pair.
+    if (stored) asm volatile("s_waitcnt vmcnt(4)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     // The compiler cannot see the wait above.  Touching this pair's query registers here makes
     // it place its own wait for them at this point, where it costs nothing; otherwise it would
     // wait at their first use, inside the tile loop, with a count that knows nothing of the
@@ -919,6 +923,7 @@ __global__ __launch_bounds__(512, 2) void flash_attn_stream_kernel(
       if (has_next) load_q(bh_next, c1, q_light);
     }
     if (c0 >= 0) run_chunk(bh, c0, b_, q_heavy);
+    stored = c0 >= 0;
     if (!has_next) break;
     bh = bh_next;
     buf ^= 1;

@@ -341,6 +341,26 @@ def test_fused_ffn_random_shapes(K, gpu_device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd", [(300, 768, 3072),    # 18 tiles of 128 x 128: the 64 x 64 tiles
+                                    (333, 200, 70),      # the same, ragged in M, N and K
+                                    (768, 2304, 768),    # 108: the 64 x 128 tiles
+                                    (1000, 1100, 130),   # the same, ragged
+                                    (1500, 3072, 100),   # 288 > the CU count: 128 x 128
+                                    (1999, 2500, 64)])
+def test_fused_ffn_small_tile_selection(K, gpu_device, dtype, M, N, Kd):
+    """Problems below the big-tile threshold on each of the three small-tile configurations
+    (picked by how many CUs 128 x 128 tiles would fill), whole and ragged, with the full epilogue."""
+    r = np.random.default_rng(M + N)
+    x = r.standard_normal((M, Kd)).astype(NP[dtype])
+    w = (r.standard_normal((Kd, N)) / np.sqrt(Kd)).astype(NP[dtype])
+    b = r.standard_normal(N).astype(NP[dtype])
+    res = r.standard_normal((M, N)).astype(NP[dtype])
+    z = K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device),
+                    residual=dev(res, gpu_device), add_gelu=True)
+    check(host(z), O.fused_ffn(x, w, b, res, add_gelu=True), dtype, f"ffn {M}x{N}x{Kd}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_lm_head_transposed_weight(K, gpu_device, dtype):
     r = np.random.default_rng(21)
     x = r.standard_normal((130, 768)).astype(NP[dtype])
