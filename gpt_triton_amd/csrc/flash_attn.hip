@@ -930,6 +930,257 @@ __global__ __launch_bounds__(512, 2) void flash_attn_stream_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Ring variant for sequences too long for the streaming kernel: fp16 storage, head size 64,
+// equal query and key lengths, no dropout.  One workgroup = 4 wavefronts = one (batch, head) x
+// 128 queries, as in the tiled kernel, but the 64-key tiles of K and V travel the way the
+// streaming kernel moves them: by direct global->LDS loads (no staging registers, no LDS store
+// instructions) into a ring of three 16 KB stages -- K tile [64][64] then V tile [64][64] halves,
+// rows of 128 bytes, the swizzles applied on the source side -- and V stays row-major and is read
+// with the transposing LDS load.  A tile is requested two steps before it is multiplied.  Two
+// workgroups per CU (200 registers; squeezed into the 168 of three wavefronts per SIMD the kernel
+// spills and is slower).  GPT-2 XL's shape (64 x 25 heads, L = 1024): 0.544 -> 0.496 ms.
+//
+// Loads retire in issue order, so "tile t has landed" is vmcnt(4): the four loads of tile t + 1
+// are the only younger ones (tile t + 2 is requested behind the barrier that follows the wait).
+// That barrier also says that every wavefront is done with tile t - 1, whose stage tile t + 2
+// then takes.  Causal structure per wavefront (first query qw0 a multiple of 32): tiles below
+// qw0 / 64 are entirely visible, tile qw0 / 64 holds the block cut by the diagonal (and, for an
+// odd 32-query chunk, one entirely visible block in front of it), later tiles are skipped -- as
+// in the streaming kernel, whose arithmetic per tile this is.
+// ---------------------------------------------------------------------------
+template <bool BLND>
+__global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
+    const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+    const _Float16* __restrict__ V, _Float16* __restrict__ O, int heads, int L, float scale) {
+  constexpr int D = 64, KS = 4, DB = 2, NS = 3;
+  constexpr int STAGE = 2 * BKEY * D * 2;  // 16 KB: K tile, then V tile
+  constexpr int V_AT = BKEY * D * 2;       // byte offset of the V tile inside a stage
+  __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ql = lane & 31, g = lane >> 5;
+  const unsigned smem_base = (unsigned)(uintptr_t)smem;
+
+  const int bh = blockIdx.x;
+  const int q_blocks = (L + BQ - 1) / BQ;
+  const int qb = q_blocks - 1 - (int)blockIdx.y;  // heavy (late) query blocks first
+  const int q0 = qb * BQ;
+  const int qw0 = q0 + wave * 32, q = qw0 + ql;
+  const bool wave_active = qw0 < L;
+  int last_q = q0 + BQ - 1;
+  if (last_q > L - 1) last_q = L - 1;
+  const int nt = last_q / BKEY + 1;  // key tiles 0..nt-1 touch this query block
+
+  // ---- queries first (the oldest loads in flight): lane (ql, g) holds d = 16 ks + 8 g + 0..7
+  h8 qf[KS];
+  {
+    const int qr = q < L ? q : L - 1;  // rows past the end are computed and never stored
+    const _Float16* qp = Q + ((int64_t)bh * L + qr) * D + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const h8*>(qp + ks * 16);
+  }
+
+  // ---- tile loads: a tile is 16 loads of 1 KB (8 rows each), K rows then V rows; wavefront w
+  // issues loads 4 w .. 4 w + 3, so wavefronts 0-1 bring K and 2-3 bring V.  Lane l fills
+  // position l % 8 of row 8 j + l / 8 with source unit (l % 8) ^ key(row): K key = (row >> 1) & 7
+  // = (4 (j & 1) + l / 16) & 7, V key = 2 (row & 3) = 2 ((l / 8) & 3).  Rows past the end of the
+  // sequence repeat the last row (their keys are masked, the values finite).
+  const bool brings_v = wave >= 2;
+  const char* src = (const char*)((brings_v ? V : K) + (int64_t)bh * L * D);
+  const int lrow = lane >> 3;
+  const unsigned unit16 =
+      brings_v ? (unsigned)(((lane & 7) ^ (2 * (lrow & 3))) << 4)
+               : (unsigned)(((lane & 7) ^ (lane >> 4)) << 4);
+  auto issue_tile = [&](int t) {
+    const unsigned dst = smem_base + (unsigned)((t % NS) * STAGE) + (unsigned)(wave * 4) * 1024u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rel = (wave & 1) * 4 + j;  // 8-row group inside the K (or V) tile
+      int row = t * BKEY + rel * 8 + lrow;
+      row = row < L ? row : L - 1;
+      const unsigned u = brings_v ? unit16 : (unit16 ^ ((unsigned)(rel & 1) << 6));
+      attn_dma16(src, (unsigned)row * 128u + u, dst + j * 1024);
+    }
+  };
+
+  // ---- LDS read offsets (bytes inside a stage) of this lane, as in the streaming kernel
+  const int tri_q = ql - 4 * g;
+  int k_off[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) k_off[ks] = ql * 128 + (((ks * 2 + g) ^ ((ql >> 1) & 7)) << 4);
+  const int sl = lane & 15, vrow = 4 * g + (sl >> 2);
+  int v_off[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int unit = 4 * i + 2 * ((lane >> 4) & 1) + ((sl & 3) >> 1);
+    v_off[i] = V_AT + vrow * 128 + ((unit ^ (2 * (vrow & 3))) << 4) + (sl & 1) * 8;
+  }
+  const float cexp = scale * 1.4426950408889634f;
+
+  f16v oacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+  float mrun = -INFINITY, den = 0.f;
+
+  // One 64-key tile in stage `buf`.  MODE 0: both 32-key blocks entirely visible; 1: block 0 cut
+  // by the diagonal, block 1 hidden (skipped: its weights are exactly 0); 2: block 0 visible,
+  // block 1 cut by the diagonal.
+  auto step = [&](auto mode_tag, const char* buf) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr int NKB = MODE == 1 ? 1 : 2;
+    // one block's K fragments at a time (16 registers, not 32)
+    f16v s[NKB];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      h8 kf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kf[ks] = *reinterpret_cast<const h8*>(buf + kb * 4096 + k_off[ks]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], s[kb], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the V^T fragments of block 0 are requested behind the score products, block 1's when
+    // block 0's products start: the LDS round trips run under the softmax arithmetic
+    h4 vlo[2][DB], vhi[2][DB];
+    auto read_v = [&](int kb) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const char* vt = buf + (kb * 32 + tt * 16) * 128;
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+          vlo[tt][i] = lds_read_tr16(vt + v_off[i]);
+          vhi[tt][i] = lds_read_tr16(vt + v_off[i] + 8 * 128);
+        }
+      }
+    };
+    read_v(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (MODE != 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s[NKB - 1][r] = 8 * (r >> 2) + (r & 3) <= tri_q ? s[NKB - 1][r] : -INFINITY;
+    }
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, s[kb][r]);
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+    const float mnew = bmax > mrun ? bmax : mrun;
+    const float mult = __builtin_amdgcn_exp2f((mrun - mnew) * cexp);
+    const float m2 = mnew * cexp;
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][r], cexp, -m2));
+        s[kb][r] = p;
+        psum += p;
+      }
+    mrun = mnew;
+    psum += __shfl_xor(psum, 32, kWave);
+    den = den * mult + psum;
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] *= mult;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      h8 vf[2][DB];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+          const h4 lo = vlo[tt][i], hi = vhi[tt][i];
+          vf[tt][i] = h8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      if (kb + 1 < NKB) {
+        __builtin_amdgcn_sched_barrier(0);
+        read_v(kb + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        h8 pf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pf[j] = (_Float16)s[kb][8 * tt + j];
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[tt][i], pf, oacc[i], 0, 0, 0);
+      }
+    }
+  };
+
+  issue_tile(0);
+  if (nt > 1) issue_tile(1);
+  const int nfull = qw0 >> 6;  // key tiles entirely below this wavefront's diagonal
+  for (int t = 0; t < nt; ++t) {
+    // tile t has landed in this wavefront's part (the queries too: they are older); behind the
+    // barrier that holds for every part, and nobody reads tile t - 1 any more
+    if (t + 1 < nt) asm volatile("s_waitcnt vmcnt(4)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (t == 0) {
+      // the compiler cannot see the wait above; touching the query registers here makes it
+      // place its own wait for them now instead of inside the first tile
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
+    }
+    if (t + 2 < nt) issue_tile(t + 2);
+    const char* buf = smem + (t % NS) * STAGE;
+    if (wave_active) {
+      if (t < nfull) step(std::integral_constant<int, 0>{}, buf);
+      else if (t == nfull) {
+        if ((qw0 & 32) == 0) step(std::integral_constant<int, 1>{}, buf);
+        else step(std::integral_constant<int, 2>{}, buf);
+      }
+    }
+  }
+
+  // ---- output, as in the streaming kernel: the two lanes of a query trade halves through the
+  // 32-lane swap and store 16 bytes each
+  const float inv = __builtin_amdgcn_rcpf(den);
+  u4 out[DB][2];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      h4 x, y;  // d = 32 i + 16 pr + 4 g + 0..3 and the same + 8
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[j] = (_Float16)(oacc[i][8 * pr + j] * inv);
+        y[j] = (_Float16)(oacc[i][8 * pr + 4 + j] * inv);
+      }
+      const u2 xd = __builtin_bit_cast(u2, x), yd = __builtin_bit_cast(u2, y);
+      const auto r0 = __builtin_amdgcn_permlane32_swap(xd[0], yd[0], false, false);
+      const auto r1 = __builtin_amdgcn_permlane32_swap(xd[1], yd[1], false, false);
+      // g = 0: own x, then the partner's x (d + 4..7); g = 1: the partner's y, then own y
+      out[i][pr] = u4{r0[0], r1[0], r0[1], r1[1]};
+    }
+  if (q < L) {
+    int64_t row_off;
+    if (BLND) {
+      const int b = bh / heads, n = bh - b * heads;
+      row_off = (((int64_t)b * L + q) * heads + n) * D;
+    } else {
+      row_off = ((int64_t)bh * L + q) * D;
+    }
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr)
+        *reinterpret_cast<u4*>(O + row_off + i * 32 + 16 * pr + 8 * g) = out[i][pr];
+  }
+}
+
 // Deals the query chunks of a sequence of L <= 320 rows to the 8 wavefronts: chunk c costs
 // c + 1 blocks; heaviest first, each to the SIMD (wavefronts w and w + 4) with the smallest
 // load so far that still has a free slot, inside the SIMD to the lighter wavefront.
@@ -1052,6 +1303,15 @@ int launch_stream_attn(const void* q, const void* k, const void* v, void* out, i
   return 0;
 }
 
+template <bool BLND>
+int launch_ring_attn(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                     int L, float scale, hipStream_t st) {
+  dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
+  hipLaunchKernelGGL(flash_attn_ring_kernel<BLND>, grid, dim3(256), 0, st, (const _Float16*)q,
+                     (const _Float16*)k, (const _Float16*)v, (_Float16*)out, heads, L, scale);
+  return 0;
+}
+
 template <int D, typename T>
 int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
              int heads, int L, int Lk, float scale, Dropout drop, bool blnd, hipStream_t st) {
@@ -1069,6 +1329,10 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
     if (L <= 320 && BN >= 64)
       return blnd ? launch_stream_attn<true>(q, k, v, out, BN, heads, L, scale, st)
                   : launch_stream_attn<false>(q, k, v, out, BN, heads, L, scale, st);
+    // sequences that do not fit the resident variant either: key tiles through the ring
+    if (resident_lds_bytes(L, D) == 0)
+      return blnd ? launch_ring_attn<true>(q, k, v, out, BN, heads, L, scale, st)
+                  : launch_ring_attn<false>(q, k, v, out, BN, heads, L, scale, st);
   }
   if (const size_t lds = resident_lds_bytes(L, D)) {
     return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)

@@ -527,6 +527,20 @@ def test_flash_attention_unequal_lengths(K, gpu_device, dtype, Lq, Lk):
         check_attention(host(z), want, v, dtype, f"attention Lq={Lq} Lk={Lk}")
 
 
+@pytest.mark.parametrize("L", [321, 383, 384, 385, 449, 700, 1025])
+def test_flash_attention_long_sequences_fp16(K, gpu_device, L):
+    """fp16, d = 64, sequences too long for the resident variant: key tiles through the ring of
+    LDS stages (direct loads, transposing reads).  Lengths either side of the 64-key tile and the
+    128-query block boundaries; both output layouts."""
+    q, k, v = attn_inputs(2, 3, L, 64, torch.float16, gaussian=True, seed=L)
+    want = O.flash_attention_v1(q, k, v)
+    args = [dev(t, gpu_device) for t in (q, k, v)]
+    z = K.flash_attention_v1(*args)
+    check(host(z), want, torch.float16, f"attention L={L}")
+    zm = K.flash_attention_v1(*args, merged_heads_layout=True)
+    assert zm.transpose(1, 2).is_contiguous() and torch.equal(z, zm)
+
+
 def test_flash_attention_xl_sequence(K, gpu_device):
     """Benchmark configuration 4 attention shape per (batch, head): L = 1024, d = 64 (the tiled kernel;
     K/V do not fit the resident variant)."""
