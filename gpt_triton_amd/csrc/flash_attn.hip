@@ -935,16 +935,16 @@ __global__ __launch_bounds__(512, 2) void flash_attn_stream_kernel(
 // equal query and key lengths, no dropout.  One workgroup = 4 wavefronts = one (batch, head) x
 // 128 queries, as in the tiled kernel, but the 64-key tiles of K and V travel the way the
 // streaming kernel moves them: by direct global->LDS loads (no staging registers, no LDS store
-// instructions) into a ring of three 16 KB stages -- K tile [64][64] then V tile [64][64] halves,
+// instructions) into a ring of four 16 KB stages -- K tile [64][64] then V tile [64][64] halves,
 // rows of 128 bytes, the swizzles applied on the source side -- and V stays row-major and is read
-// with the transposing LDS load.  A tile is requested two steps before it is multiplied.  Two
-// workgroups per CU (200 registers; squeezed into the 168 of three wavefronts per SIMD the kernel
-// spills and is slower).  GPT-2 XL's shape (64 x 25 heads, L = 1024): 0.544 -> 0.496 ms.
+// with the transposing LDS load.  A tile is requested three steps before its P.V products.  Two
+// workgroups per CU (198 registers; squeezed into the 168 of three wavefronts per SIMD the kernel
+// spills and is slower).  GPT-2 XL's shape (64 x 25 heads, L = 1024): 0.544 -> 0.489 ms.
 //
-// Loads retire in issue order, so "tile t has landed" is vmcnt(4): the four loads of tile t + 1
-// are the only younger ones (tile t + 2 is requested behind the barrier that follows the wait).
-// That barrier also says that every wavefront is done with tile t - 1, whose stage tile t + 2
-// then takes.  Causal structure per wavefront (first query qw0 a multiple of 32): tiles below
+// Loads retire in issue order, so "tiles t and t + 1 have landed" is vmcnt(4): the four loads of
+// tile t + 2 are the only younger ones (tile t + 3 is requested behind the barrier that follows
+// the wait).  That barrier also says that every wavefront is done with tile t - 1, whose stage
+// tile t + 3 then takes.  Causal structure per wavefront (first query qw0 a multiple of 32): tiles below
 // qw0 / 64 are entirely visible, tile qw0 / 64 holds the block cut by the diagonal (and, for an
 // odd 32-query chunk, one entirely visible block in front of it), later tiles are skipped -- as
 // in the streaming kernel, whose arithmetic per tile this is.
@@ -953,7 +953,7 @@ template <bool BLND>
 __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
     const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     const _Float16* __restrict__ V, _Float16* __restrict__ O, int heads, int L, float scale) {
-  constexpr int D = 64, KS = 4, DB = 2, NS = 3;
+  constexpr int D = 64, KS = 4, DB = 2, NS = 4;
   constexpr int STAGE = 2 * BKEY * D * 2;  // 16 KB: K tile, then V tile
   constexpr int V_AT = BKEY * D * 2;       // byte offset of the V tile inside a stage
   __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE];
@@ -1025,14 +1025,13 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
   float mrun = -INFINITY, den = 0.f;
 
-  // One 64-key tile in stage `buf`.  MODE 0: both 32-key blocks entirely visible; 1: block 0 cut
-  // by the diagonal, block 1 hidden (skipped: its weights are exactly 0); 2: block 0 visible,
-  // block 1 cut by the diagonal.
-  auto step = [&](auto mode_tag, const char* buf) {
-    constexpr int MODE = decltype(mode_tag)::value;
-    constexpr int NKB = MODE == 1 ? 1 : 2;
-    // one block's K fragments at a time (16 registers, not 32)
-    f16v s[NKB];
+  // A 64-key tile is worked on in three parts.  MODE 0: both 32-key blocks entirely visible; 1:
+  // block 0 cut by the diagonal, block 1 hidden (skipped: its weights are exactly 0); 2: block 0
+  // visible, block 1 cut by the diagonal.
+  f16v s[2];  // S^T of the tile whose softmax comes next
+  // scores(MODE, stage): S^T = K . Q^T, one block's K fragments at a time (16 registers, not 32)
+  auto scores = [&](auto mode_tag, const char* buf) {
+    constexpr int NKB = decltype(mode_tag)::value == 1 ? 1 : 2;
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
       h8 kf[KS];
@@ -1046,22 +1045,26 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
         s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], s[kb], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // the V^T fragments of block 0 are requested behind the score products, block 1's when
-    // block 0's products start: the LDS round trips run under the softmax arithmetic
-    h4 vlo[2][DB], vhi[2][DB];
-    auto read_v = [&](int kb) {
+  };
+  // V^T fragments of one 32-key block of the tile in `buf`
+  h4 vlo[2][DB], vhi[2][DB];
+  auto read_v = [&](const char* buf, int kb) {
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const char* vt = buf + (kb * 32 + tt * 16) * 128;
+    for (int tt = 0; tt < 2; ++tt) {
+      const char* vt = buf + (kb * 32 + tt * 16) * 128;
 #pragma unroll
-        for (int i = 0; i < DB; ++i) {
-          vlo[tt][i] = lds_read_tr16(vt + v_off[i]);
-          vhi[tt][i] = lds_read_tr16(vt + v_off[i] + 8 * 128);
-        }
+      for (int i = 0; i < DB; ++i) {
+        vlo[tt][i] = lds_read_tr16(vt + v_off[i]);
+        vhi[tt][i] = lds_read_tr16(vt + v_off[i] + 8 * 128);
       }
-    };
-    read_v(0);
-    __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // softmax(MODE): mask, running max, P = exp(S - max) summed into the denominator and rounded to
+  // fp16 (pf: the second operand of the P.V products, [block][16-key step]), accumulator rescaled
+  h8 pf[2][2];
+  auto softmax = [&](auto mode_tag) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr int NKB = MODE == 1 ? 1 : 2;
     if constexpr (MODE != 0) {
 #pragma unroll
       for (int r = 0; r < 16; ++r)
@@ -1080,11 +1083,13 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][r], cexp, -m2));
-        s[kb][r] = p;
-        psum += p;
-      }
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][8 * tt + j], cexp, -m2));
+          psum += p;
+          pf[kb][tt][j] = (_Float16)p;
+        }
     mrun = mnew;
     psum += __shfl_xor(psum, 32, kWave);
     den = den * mult + psum;
@@ -1092,7 +1097,11 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
     for (int i = 0; i < DB; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[i][r] *= mult;
-    __builtin_amdgcn_sched_barrier(0);
+  };
+  // weighted(MODE, stage): O^T += V^T . P^T; block 0's V^T fragments are in registers already,
+  // block 1's are requested when block 0's products start
+  auto weighted = [&](auto mode_tag, const char* buf) {
+    constexpr int NKB = decltype(mode_tag)::value == 1 ? 1 : 2;
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
       h8 vf[2][DB];
@@ -1105,28 +1114,39 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
         }
       if (kb + 1 < NKB) {
         __builtin_amdgcn_sched_barrier(0);
-        read_v(kb + 1);
+        read_v(buf, kb + 1);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        h8 pf;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pf[j] = (_Float16)s[kb][8 * tt + j];
+      for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int i = 0; i < DB; ++i)
-          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[tt][i], pf, oacc[i], 0, 0, 0);
-      }
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[tt][i], pf[kb][tt], oacc[i], 0, 0, 0);
     }
   };
 
+  // The order inside a wavefront: softmax of tile t, THEN the score products of tile t + 1, then
+  // the P.V products of tile t.  The matrix pipe works through them in that order, so the scores
+  // of tile t + 1 are ready when the softmax of tile t + 1 starts (they only queue behind nothing,
+  // and the P.V products of tile t run under that softmax) instead of queueing behind the P.V
+  // products.  Needs tile t + 1 published one step earlier: four stages, tile t + 3 requested at
+  // step t.
+  const int nfull = qw0 >> 6;  // key tiles entirely below this wavefront's diagonal
+  const int diag_mode = (qw0 & 32) == 0 ? 1 : 2;
+  auto stage_of = [&](int t) { return (const char*)smem + (t % NS) * STAGE; };
+  auto scores_of = [&](int t) {  // t <= nfull
+    if (t < nfull) scores(std::integral_constant<int, 0>{}, stage_of(t));
+    else if (diag_mode == 1) scores(std::integral_constant<int, 1>{}, stage_of(t));
+    else scores(std::integral_constant<int, 2>{}, stage_of(t));
+  };
   issue_tile(0);
   if (nt > 1) issue_tile(1);
-  const int nfull = qw0 >> 6;  // key tiles entirely below this wavefront's diagonal
+  if (nt > 2) issue_tile(2);
   for (int t = 0; t < nt; ++t) {
-    // tile t has landed in this wavefront's part (the queries too: they are older); behind the
-    // barrier that holds for every part, and nobody reads tile t - 1 any more
-    if (t + 1 < nt) asm volatile("s_waitcnt vmcnt(4)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // tiles t and t + 1 have landed in this wavefront's part (the queries too: they are older;
+    // the four loads of tile t + 2 are the only younger ones); behind the barrier that holds for
+    // every part, and nobody reads tile t - 1 any more
+    if (t + 2 < nt) asm volatile("s_waitcnt vmcnt(4)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (t == 0) {
       // the compiler cannot see the wait above; touching the query registers here makes it
@@ -1134,13 +1154,25 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
     }
-    if (t + 2 < nt) issue_tile(t + 2);
-    const char* buf = smem + (t % NS) * STAGE;
-    if (wave_active) {
-      if (t < nfull) step(std::integral_constant<int, 0>{}, buf);
-      else if (t == nfull) {
-        if ((qw0 & 32) == 0) step(std::integral_constant<int, 1>{}, buf);
-        else step(std::integral_constant<int, 2>{}, buf);
+    if (t + 3 < nt) issue_tile(t + 3);
+    if (wave_active && t <= nfull) {
+      const char* buf = stage_of(t);
+      if (t == 0) scores_of(0);
+      read_v(buf, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (t < nfull) {
+        softmax(std::integral_constant<int, 0>{});
+        __builtin_amdgcn_sched_barrier(0);
+        scores_of(t + 1);
+        weighted(std::integral_constant<int, 0>{}, buf);
+      } else if (diag_mode == 1) {
+        softmax(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+        weighted(std::integral_constant<int, 1>{}, buf);
+      } else {
+        softmax(std::integral_constant<int, 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+        weighted(std::integral_constant<int, 2>{}, buf);
       }
     }
   }
