@@ -67,10 +67,12 @@ __device__ __forceinline__ h8 zero_h8() {
   return z;
 }
 
-// D = head size.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
+// D = head size of the LDS tiles.  LDS per stage: K tile [64][D] (16-byte chunk c of row r at
 // position c ^ (r&7)) and V^T tile [D][64] (8-byte unit u of row d at position
-// u ^ ((d>>1)&15)).
-template <int D, typename T, bool BLND, bool DROP, bool UNEQ>
+// u ^ ((d>>1)&15)).  DG = head size of the tensors in memory: 16 and 32 run on the D = 64
+// staging layout (columns at or past DG are written as zeros, never read from memory) with
+// only DG / 16 k-steps of q . k and one 32-row block of O^T.
+template <int D, typename T, bool BLND, bool DROP, bool UNEQ, int DG = D>
 __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     T* __restrict__ O, int heads, int L, int Lk_arg, float scale, DropoutArgs drop) {
@@ -81,8 +83,9 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   // read the last row again instead (no select per load).
   const int Lk = UNEQ ? Lk_arg : L;
   constexpr int CH = D / 8;             // 16-byte chunks per row
-  constexpr int KS = D / 16;            // MFMA k-steps over the head dim
-  constexpr int DB = D / 32;            // 32-row blocks of O^T
+  static_assert(DG == D || (D == 64 && (DG == 16 || DG == 32) && UNEQ), "small heads: D = 64");
+  constexpr int KS = DG / 16;           // MFMA k-steps over the head dim
+  constexpr int DB = (DG + 31) / 32;    // 32-row blocks of O^T
   constexpr int K_BYTES = BKEY * D * 2;
   constexpr int STAGE = 2 * K_BYTES;
   constexpr int K_LD = BKEY * CH / 128; // K chunks per staging thread
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   // heavy (late) query blocks first so the tail of the grid is light
   const int qb = q_blocks - 1 - (int)blockIdx.y;
   const int q0 = qb * BQ;
-  const int64_t base = (int64_t)bh * L * D, kv_base = (int64_t)bh * Lk * D;
+  const int64_t base = (int64_t)bh * L * DG, kv_base = (int64_t)bh * Lk * DG;
   const T* Qp = Q + base;
   const T* Kp = K + kv_base;
   const T* Vp = V + kv_base;
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   h8 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
-    qf[ks] = q < L ? Ld8<T>::load(Qp + (int64_t)q * D + ks * 16 + g * 8) : zero_h8();
+    qf[ks] = q < L ? Ld8<T>::load(Qp + (int64_t)q * DG + ks * 16 + g * 8) : zero_h8();
 
   int last_q = q0 + BQ - 1;
   if (last_q > L - 1) last_q = L - 1;
@@ -151,7 +154,8 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     for (int i = 0; i < NLD; ++i) {
       int row = k0 + srow[i];
       if constexpr (UNEQ) {
-        dst[i] = row < Lk ? Ld8<T>::load(sp + (int64_t)row * D + scol[i]) : zero_h8();
+        const bool there = DG < D ? (row < Lk && scol[i] < DG) : row < Lk;
+        dst[i] = there ? Ld8<T>::load(sp + (int64_t)row * DG + scol[i]) : zero_h8();
       } else {
         row = row < L ? row : L - 1;
         dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
@@ -330,15 +334,16 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     int64_t row_off;
     if (BLND) {
       const int b = bh / heads, n = bh - b * heads;
-      row_off = (((int64_t)b * L + q) * heads + n) * D;
+      row_off = (((int64_t)b * L + q) * heads + n) * DG;
     } else {
-      row_off = base + (int64_t)q * D;
+      row_off = base + (int64_t)q * DG;
     }
 #pragma unroll
     for (int i = 0; i < DB; ++i)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         const int d = i * 32 + 8 * rg + 4 * g;
+        if (DG < 32 && d >= DG) continue;
         if constexpr (sizeof(T) == 2) {
           h4 o;
 #pragma unroll
@@ -1264,12 +1269,12 @@ int launch_resident(const void* q, const void* k, const void* v, void* out, int6
   return 0;
 }
 
-template <int D, typename T, bool BLND, bool DROP, bool UNEQ>
+template <int D, typename T, bool BLND, bool DROP, bool UNEQ, int DG = D>
 int launch_tiled_as(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
                     int L, int Lk, float scale, DropoutArgs drop, hipStream_t st) {
   dim3 grid((unsigned)BN, (unsigned)((L + BQ - 1) / BQ));
   constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V^T tile
-  auto kern = flash_attn_kernel<D, T, BLND, DROP, UNEQ>;
+  auto kern = flash_attn_kernel<D, T, BLND, DROP, UNEQ, DG>;
   static bool attr_done = false;  // idempotent; a race only repeats the call
   if (!attr_done && lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1374,15 +1379,34 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
               : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st);
 }
 
+// Head sizes 16 and 32: the tiled kernel on its 64-wide staging layout, reading the tensors at
+// their own row pitch (the variant that knows both sequence lengths serves equal ones too).
+template <int DG, typename T>
+int launch_small_head(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                      int L, int Lk, float scale, Dropout drop, bool blnd, hipStream_t st) {
+  const DropoutArgs da = {drop.p, (unsigned)drop.seed, (unsigned)(drop.seed >> 32)};
+  if (drop.p > 0.f)
+    return blnd ? launch_tiled_as<64, T, true, true, true, DG>(q, k, v, out, BN, heads, L, Lk,
+                                                               scale, da, st)
+                : launch_tiled_as<64, T, false, true, true, DG>(q, k, v, out, BN, heads, L, Lk,
+                                                                scale, da, st);
+  return blnd ? launch_tiled_as<64, T, true, false, true, DG>(q, k, v, out, BN, heads, L, Lk,
+                                                              scale, da, st)
+              : launch_tiled_as<64, T, false, false, true, DG>(q, k, v, out, BN, heads, L, Lk,
+                                                               scale, da, st);
+}
+
 template <typename T>
 int launch_t(const void* q, const void* k, const void* v, void* out, int64_t BN,
              int heads, int L, int Lk, int d, float scale, Dropout drop, bool blnd, hipStream_t st) {
   switch (d) {
+    case 16: return launch_small_head<16, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
+    case 32: return launch_small_head<32, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
     case 64: return launch_d<64, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
     case 128: return launch_d<128, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
     case 256: return launch_d<256, T>(q, k, v, out, BN, heads, L, Lk, scale, drop, blnd, st);
     default:
-      set_error("flash_attn: head size %d not built (64, 128 and 256 are)", d);
+      set_error("flash_attn: head size %d not built (16, 32, 64, 128 and 256 are)", d);
       return -2;
   }
 }

@@ -346,13 +346,6 @@ def flash_attention_v1(q, k, v, dropout_prob=0.0, *, merged_heads_layout=False):
     dev = _on_gpu(q, k, v)
     code = _dtype_code(q, "flash_attention_v1")
     scale = 1 / math.sqrt(H)
-    if H < 64:
-        # The kernels are built for head sizes 64, 128 and 256.  Zero columns add nothing to
-        # q . k and give zero output columns, so 16 and 32 run as 64 with the scale of the true
-        # size and the padding cut off again (two small copies; GPT-2 itself never has d < 64).
-        pad = lambda t: torch.nn.functional.pad(t, (0, 64 - H)).contiguous()
-        out = _flash(pad(q), pad(k), pad(v), scale, dropout_prob, merged_heads_layout, dev, code)
-        return out[..., :H] if merged_heads_layout else out[..., :H].contiguous()
     return _flash(q, k, v, scale, dropout_prob, merged_heads_layout, dev, code)
 
 

@@ -223,7 +223,9 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
  *
  * Replaces flash_attention_v1(q, k, v, dropout_prob) -> kernels.py:477-525 and
  * flash_attention_v1_kernel -> kernels.py:375-474.
- *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 64, 128 or 256
+ *   q [B][N][Lq][d]    k, v [B][N][Lk][d]    d = 16, 32, 64, 128 or 256 (the reference's
+ *   set, kernels.py:490; 16 and 32 are read at their own row pitch and multiplied on the
+ *   64-wide tiles of the d = 64 kernel, the missing columns being zeros in LDS only)
  * Lq != Lk behaves as in the reference (kernels.py:421-436): the mask is "key <= query" from the
  * top left, nothing else, and the last 64-key tile is filled up with zero rows.  So with Lq < Lk
  * the keys past the last query play no part, and with Lq > Lk a query at or past Lk attends to all

@@ -487,14 +487,24 @@ def test_flash_attention_merged_heads_layout(K, gpu_device, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("D", [16, 32])
 def test_flash_attention_small_heads(K, gpu_device, dtype, D):
-    """Head sizes 16 and 32 (accepted by the reference, kernels.py:490) run zero padded to 64."""
-    q, k, v = attn_inputs(2, 3, 130, D, dtype, gaussian=True, seed=9)
-    z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
-    assert z.shape == (2, 3, 130, D) and z.is_contiguous()
-    check_attention(host(z), O.flash_attention_v1(q, k, v), v, dtype, f"d={D}")
-    zm = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
-                              merged_heads_layout=True)
-    assert np.array_equal(host(zm), host(z))
+    """Head sizes 16 and 32 (accepted by the reference, kernels.py:490), read at their own row
+    pitch: equal and unequal sequence lengths, both output layouts, dropout."""
+    for Lq, Lk in ((130, 130), (1, 1), (64, 64), (70, 150), (150, 70)):
+        r = np.random.default_rng(9 + Lq + 3 * Lk)
+        q = r.standard_normal((2, 3, Lq, D)).astype(NP[dtype])
+        k, v = (r.standard_normal((2, 3, Lk, D)).astype(NP[dtype]) for _ in range(2))
+        z = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device))
+        assert z.shape == (2, 3, Lq, D) and z.is_contiguous()
+        check_attention(host(z), O.flash_attention_v1(q, k, v), v, dtype, f"d={D} {Lq}x{Lk}")
+        zm = K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                                  merged_heads_layout=True)
+        assert zm.transpose(1, 2).is_contiguous()
+        assert np.array_equal(host(zm), host(z))
+    q, k, v = attn_inputs(1, 2, 100, D, dtype, gaussian=True, seed=10)
+    z = host(K.flash_attention_v1(dev(q, gpu_device), dev(k, gpu_device), dev(v, gpu_device),
+                                  dropout_prob=0.2))
+    want = O.flash_attention_v1(q, k, v, dropout_prob=0.2)
+    check_attention(z, want, v.astype(np.float32) / 0.8, dtype, f"d={D} dropout")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
