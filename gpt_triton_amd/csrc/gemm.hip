@@ -1085,8 +1085,9 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < MB; ++j) {
-          const int q = i * MB + j;
+        for (int jj = 0; jj < MB; ++jj) {
+          const int q = i * MB + jj;
+          const int j = (i & 1) ? MB - 1 - jj : jj;  // one operand changes per MFMA
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
                                                              0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
@@ -1363,8 +1364,9 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < MB; ++j) {
-          const int q = i * MB + j;
+        for (int jj = 0; jj < MB; ++jj) {
+          const int q = i * MB + jj;
+          const int j = (i & 1) ? MB - 1 - jj : jj;  // one operand changes per MFMA
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
                                                              0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
