@@ -201,6 +201,38 @@ __device__ __forceinline__ void bias_to_f32(const P4 (&raw)[NB][4], f4 (&bias_r)
       for (int e = 0; e < 4; ++e) bias_r[i][g][e] = (float)raw[i][g][e];
 }
 
+// The same for the accumulators of v_mfma_f32_16x16x32 (the streaming kernels): of a 32 x 32
+// block a lane holds four quads, (mh, nh) -> row 16 mh + lane % 16, columns 16 nh + 4 (lane / 16)
+// + 0..3, so two bias quads per block: [i][nh] -> columns nw0 + 32 i + 16 nh + 4 (lane / 16) + 0..3.
+template <typename T, int NB>
+__device__ __forceinline__ void load_bias16(const EpiDev& ep, int nw0, int lq,
+                                            typename Pack4<T>::type (&raw)[NB][2]) {
+  typedef typename Pack4<T>::type P4;
+  if (ep.bias) {
+    const T* bp = (const T*)ep.bias + (nw0 + lq * 4);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int nh = 0; nh < 2; ++nh) raw[i][nh] = *reinterpret_cast<const P4*>(bp + i * 32 + nh * 16);
+  } else {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int nh = 0; nh < 2; ++nh)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) raw[i][nh][e] = 0;
+  }
+}
+template <typename P4, int NB>
+__device__ __forceinline__ void bias_to_f32_16(const P4 (&raw)[NB][2], f4 (&bias_r)[NB][2]) {
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int nh = 0; nh < 2; ++nh)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bias_r[i][nh][e] = (float)raw[i][nh][e];
+}
+
 constexpr int EP_STRIDE = 64 * 4 + 16;  // bytes of one staged epilogue row (64 fp32 + pad)
 constexpr int EP_SLAB = 32 * EP_STRIDE; // one wavefront's staging slab
 
@@ -351,14 +383,20 @@ __device__ __forceinline__ void store_wave_tile_v(f16v (&acc)[NB][MB], const Epi
 // the one rounding, so those epilogues keep the fp32 slabs.
 // bias_r[i][g] = bias of the lane's 4 columns nw0 + 32 i + 8 g + 4 (lane / 32) + 0..3.
 // (NB / 2) * MB * 4 stores per lane.
-template <int MB, int NB, bool QKV, bool GELU>
-__device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+// L16: the accumulators are those of v_mfma_f32_16x16x32 -- acc[2 NB][2 MB] of 4 floats, and of
+// the 32 x 32 block (i, j) a lane holds the quads (mh, nh) = acc[2 i + nh][2 j + mh]: row
+// 16 mh + lane % 16, columns 16 nh + 4 (lane / 16) + 0..3, bias_r[i][nh] (see load_bias16).  Only
+// where a quad comes from and where it lands in the slab differs; the slab and what leaves it do not.
+template <int MB, int NB, bool QKV, bool GELU, bool L16 = false, typename Acc, typename Bias>
+__device__ __forceinline__ void store_wave_tile_h(Acc& acc, const Bias& bias_r,
                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
                                                   char* slab, int lane) {
   static_assert(NB % 2 == 0, "wave tile must be a multiple of 64 columns");
   // key (row >> 1) & 7: the 32 rows x 2 lanes of one 8-byte write then cover 16 distinct
   // 16-byte slots of the 256-byte bank window twice -- the minimum for 512 bytes
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  const int lq = lane >> 4;
+  const int frow = L16 ? (lane & 15) : (lane & 31), fhalf = L16 ? (lq & 1) : (lane >> 5);
+  const int fkey = (frow >> 1) & 7;  // rows 16 apart share a key
   const int rrow = lane >> 3, runit = lane & 7;
   const int rkey = rrow >> 1;  // key of row 8 rr + rrow = rkey ^ 4 (rr & 1)
   _Float16* qkv_col[NB / 2];
@@ -384,14 +422,19 @@ __device__ __forceinline__ void store_wave_tile_h(f16v (&acc)[NB][MB], const f4 
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int i = i2 * 2 + ii;
+          const int mh = g >> 1, nh = g & 1;  // L16: quad g = (mh, nh)
           h4 o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+            float z;
+            if constexpr (L16) z = acc[2 * i + nh][2 * j + mh][e] + bias_r[i][nh][e];
+            else z = acc[i][j][4 * g + e] + bias_r[i][g][e];
             if (GELU) z = gelu_new(z);
             o[e] = (_Float16)z;
           }
-          *reinterpret_cast<h4*>(slab + frow * 128 + (((ii * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+          const int row = L16 ? 16 * mh + frow : frow;
+          const int grp = L16 ? 2 * nh + (lq >> 1) : g;  // 8-column group of the quad
+          *reinterpret_cast<h4*>(slab + row * 128 + (((ii * 4 + grp) ^ fkey) << 4) + fhalf * 8) = o;
         }
       // all four reads first: the stores are assembly with a memory clobber, which no LDS
       // read may cross, so reading inside the store loop would expose one LDS latency per store
@@ -490,12 +533,14 @@ __device__ __forceinline__ void store_wave_tile_rl(f16v (&acc)[NB][MB], const f4
 // starts: the second half's 8 loads.  Younger than the second half's loads when band 2 starts: the
 // 8 stores of bands 0 and 1 and, if `refilled`, the 8 operand loads `mid` issued.
 template <int MB, int NB, bool GELU, typename Mid>
-__device__ __forceinline__ void store_wave_tile_rs(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+__device__ __forceinline__ void store_wave_tile_rs(f4 (&acc)[2 * NB][2 * MB], const f4 (&bias_r)[NB][2],
                                                    const EpiDev& ep, int64_t mw0, int nw0, int N,
                                                    const char* res_lo, const char* res_hi,
                                                    char* slab, int lane, bool refilled, Mid&& mid) {
   static_assert(MB == 4 && NB == 2, "128 x 64 sub-tile");
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  // accumulators of v_mfma_f32_16x16x32: quad (mh, nh) of the 32 x 32 block (i, j), see
+  // store_wave_tile_h<L16>
+  const int frow = lane & 15, lq = lane >> 4, fhalf = lq & 1, fkey = (frow >> 1) & 7;
   const int rrow = lane >> 3, runit = lane & 7, rkey = rrow >> 1;
   const unsigned lane_byte_off = ((unsigned)rrow * (unsigned)N + runit * 8) * 2u;
 #pragma unroll
@@ -511,20 +556,25 @@ __device__ __forceinline__ void store_wave_tile_rs(f16v (&acc)[NB][MB], const f4
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        r[i][g] = *reinterpret_cast<const h4*>(rb + (((i * 4 + g) ^ fkey) << 4));
+      for (int g = 0; g < 4; ++g) {
+        const int mh = g >> 1, nh = g & 1;
+        r[i][g] = *reinterpret_cast<const h4*>(rb + mh * 16 * 128 +
+                                               (((i * 4 + 2 * nh + (lq >> 1)) ^ fkey) << 4));
+      }
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const int mh = g >> 1, nh = g & 1;
         h4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float z = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          float z = acc[2 * i + nh][2 * j + mh][e] + bias_r[i][nh][e];
           if (GELU) z = gelu_new(z);
           o[e] = (_Float16)(z + (float)r[i][g][e]);
         }
-        *reinterpret_cast<h4*>(slab + frow * 128 + (((i * 4 + g) ^ fkey) << 4) + fhalf * 8) = o;
+        *reinterpret_cast<h4*>(slab + (16 * mh + frow) * 128 +
+                               (((i * 4 + 2 * nh + (lq >> 1)) ^ fkey) << 4) + fhalf * 8) = o;
       }
     h8 vv[4];
 #pragma unroll
@@ -890,11 +940,13 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
 // residual, no dropout: the launcher sends everything else to gemm_kernel.
 // ---------------------------------------------------------------------------
 template <int MB, int NB, typename T, bool QKV, bool GELU>
-__device__ __forceinline__ void store_wave_tile32(f16v (&acc)[NB][MB], const f4 (&bias_r)[NB][4],
+__device__ __forceinline__ void store_wave_tile32(f4 (&acc)[2 * NB][2 * MB], const f4 (&bias_r)[NB][2],
                                                   const EpiDev& ep, int64_t mw0, int nw0, int N,
                                                   char* slab, int lane) {
   typedef typename Pack4<T>::type P4;
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
+  // accumulators of v_mfma_f32_16x16x32: quad (mh, nh) of the 32 x 32 block (i, j) = row
+  // 16 mh + lane % 16, columns 16 nh + 4 (lane / 16) + 0..3
+  const int frow = lane & 15, lq = lane >> 4, fkey = (frow >> 1) & 7;
   const int rrow = lane >> 3, runit = lane & 7;
   T* qkv_col[NB];
   unsigned b0 = 0, l0 = 0;
@@ -916,13 +968,14 @@ __device__ __forceinline__ void store_wave_tile32(f16v (&acc)[NB][MB], const f4 
     for (int i = 0; i < NB; ++i) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const int mh = g >> 1, nh = g & 1;
         f4 z;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          z[e] = acc[i][j][4 * g + e] + bias_r[i][g][e];
+          z[e] = acc[2 * i + nh][2 * j + mh][e] + bias_r[i][nh][e];
           if (GELU) z[e] = gelu_new(z[e]);
         }
-        *reinterpret_cast<f4*>(slab + frow * 128 + (((g * 2 + fhalf) ^ fkey) << 4)) = z;
+        *reinterpret_cast<f4*>(slab + (16 * mh + frow) * 128 + (((4 * nh + lq) ^ fkey) << 4)) = z;
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
@@ -1031,19 +1084,34 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     for (int n = 0; n < B_IT; ++n) issue_b(stage, b_src(n0, k, n), n);
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
-  const int a_row_off = (wm * TM + frow) * ROWB;
-  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
-  h8 af[2][MB], bf[2][NB];
-  auto read_frags = [&](int stage, int ks, int slot) __attribute__((always_inline)) {
+  // Fragments of v_mfma_f32_16x16x32_f16: a lane supplies row lane % 16 of a block of 16 rows and
+  // the 8 halves of 16-byte unit lane / 16 of a 32-wide k-step.  (Which k goes to which lane group
+  // is free as long as both operands agree: k is summed over.)  16 consecutive lanes read 16
+  // consecutive rows at one unit, as with the 32-row fragments of the small-tile kernel: no bank
+  // conflicts.
+  const int lrow = lane & 15, lq = lane >> 4, fkey = (lrow >> 1) & 7;
+  const int a_row_off = (wm * TM + lrow) * ROWB;
+  const int b_row_off = BM * ROWB + (wn * TN + lrow) * ROWB;
+  // A slice = one 32-wide k-step s times one half h of the sub-tile's rows: 4 A blocks (af; a
+  // block's register takes the next slice's block as soon as its four MFMAs are issued) times 4 B
+  // blocks (bf[s], good for both halves of step s).
+  static_assert(TM == 128 && TN == 64, "128 x 64 sub-tiles");
+  h8 af[4], bf[2][4];
+  auto frag_a = [&](const char* st, int h, int jl, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(st + a_row_off + (h * 64 + jl * 16) * ROWB +
+                                        (((s * 4 + lq) ^ fkey) << 4));
+  };
+  auto frag_b = [&](const char* st, int i, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(st + b_row_off + i * 16 * ROWB +
+                                        (((s * 4 + lq) ^ fkey) << 4));
+  };
+  // the fragments of a k-tile's first slice
+  auto read_first = [&](int stage) __attribute__((always_inline)) {
     const char* st = smem + stage * STAGE;
-    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
-    for (int j = 0; j < MB; ++j)
-      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
+    for (int jl = 0; jl < 4; ++jl) af[jl] = frag_a(st, 0, jl, 0);
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
+    for (int i = 0; i < 4; ++i) bf[0][i] = frag_b(st, i, 0);
   };
 
   int vp = blockIdx.x;
@@ -1053,7 +1121,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
   issue(1, m0, n0, 1);
   wait_vmcnt<LPT>();
   asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
+  read_first(0);
   int stage = 0;           // stage of the k-tile being multiplied
   bool prev_stored = false;  // this wavefront stored a tile right before the current one
 
@@ -1066,44 +1134,48 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     const int nw0 = n0 + wn * TN;
     const bool wave_stores = nw0 < N;  // else this wavefront's 64 columns lie past the edge
 
-    f16v acc[NB][MB];
+    // acc[i][j] = the 16 x 16 block of columns 16 i.., rows 16 j.. of the sub-tile: a lane holds
+    // row lane % 16 and the 4 columns 4 (lane / 16) + 0..3
+    f4 acc[2 * NB][2 * MB];
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
+    for (int i = 0; i < 2 * NB; ++i)
 #pragma unroll
-      for (int j = 0; j < MB; ++j)
+      for (int j = 0; j < 2 * MB; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    // One k-slice: the eight MFMAs on fragment slot `slot`.  Behind the first six of them, one
-    // each, go the fragment reads of slice `rks` of `rstage` into the other slot, in the order
-    // the next slice uses them: a read issued in the shadow of an MFMA costs no issue time,
-    // six of them in front of the MFMAs idle the pipe whenever both wavefronts of a SIMD read
-    // at once (behind every barrier).  `extra(q)` runs behind MFMA q.
-    auto slice = [&](int slot, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+    // One slice, a quarter of a k-tile: 16 MFMAs of 16 x 16 x 32 in eight pairs (a pair takes the
+    // matrix pipe as long as one 32 x 32 x 16, and this shape draws less power for the same
+    // products: on random operands the chip holds a higher clock).  Behind the pairs, one each, go
+    // the fragment reads for slice `rks` of `rstage`: a read issued in the shadow of an MFMA costs
+    // no issue time, a burst of them in front of the MFMAs idles the pipe whenever both wavefronts
+    // of a SIMD read at once (behind every barrier).  `extra(q)` runs behind pair q.
+    auto slice = [&](int, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+      // this slice is t = rks - 1 (mod 4): k-step s = t / 2, row half h = t % 2
+      const int t = (rks + 3) & 3, s = t >> 1, h = t & 1;
       const char* st = smem + rstage * STAGE;
-      const int choff = ((rks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+      for (int q = 0; q < 8; ++q) {
+        const int jl = q >> 1;
 #pragma unroll
-        for (int jj = 0; jj < MB; ++jj) {
-          const int q = i * MB + jj;
-          const int j = (i & 1) ? MB - 1 - jj : jj;  // one operand changes per MFMA
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
-                                                             0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          if (fetch) {
-            if (q == 0)
-              bf[slot ^ 1][0] = *reinterpret_cast<const h8*>(st + b_row_off + choff);
-            else if (q <= MB)
-              af[slot ^ 1][q - 1] =
-                  *reinterpret_cast<const h8*>(st + a_row_off + (q - 1) * 32 * ROWB + choff);
-            else if (q < MB + NB)
-              bf[slot ^ 1][q - MB] =
-                  *reinterpret_cast<const h8*>(st + b_row_off + (q - MB) * 32 * ROWB + choff);
-          }
-          extra(q);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int p = 0; p < 2; ++p) {
+          const int ii = (q & 1) * 2 + p;
+          const int i = (jl & 1) ? 3 - ii : ii;  // one operand changes per MFMA
+          acc[i][4 * h + jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[s][i], af[jl],
+                                                                      acc[i][4 * h + jl], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (fetch) {
+          // behind an A block's second pair: the same block of the next slice.  Behind the first
+          // pairs: the B blocks of k-step 1 (during slice 1) or of the published k-tile's k-step 0
+          // (during slice 3); each B set is idle while it is written.
+          if (q & 1) af[jl] = frag_a(st, rks & 1, jl, rks >> 1);
+          else if (t == 1) bf[1][jl] = frag_b(st, jl, 1);
+          else if (t == 3) bf[0][jl] = frag_b(st, jl, 0);
+        }
+        extra(q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     };
     auto nothing = [](int) __attribute__((always_inline)) {};
     // A refill dealt one load behind every MFMA of one slice arrives at the texture unit faster
@@ -1163,24 +1235,24 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     // falls behind those loads.  The next tile's first fragments are read after the epilogue.
     // fp16: requested a whole k-tile before it is needed; fp32 (twice the registers): in front
     // of the last slice
-    typename Pack4<T>::type bias_raw[NB][4];
+    typename Pack4<T>::type bias_raw[NB][2];
     if constexpr (sizeof(T) == 2) {
-      if (wave_stores) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+      if (wave_stores) load_bias16<T, NB>(ep, nw0, lq, bias_raw);
     }
     __builtin_amdgcn_sched_barrier(0);
     first_slices(with_b_half);
     if (has_next) publish_next(false);
     if constexpr (sizeof(T) == 4) {
-      if (wave_stores) load_bias<T, NB>(ep, nw0, fhalf, bias_raw);
+      if (wave_stores) load_bias16<T, NB>(ep, nw0, lq, bias_raw);
     }
     __builtin_amdgcn_sched_barrier(0);
     slice(1, false, 0, 0, nothing);
-    f4 bias_r[NB][4];
-    bias_to_f32(bias_raw, bias_r);
+    f4 bias_r[NB][2];
+    bias_to_f32_16(bias_raw, bias_r);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
+      for (int g = 0; g < 2; ++g) asm volatile("" : "+v"(bias_r[i][g]));
     if (has_next) issue(stage, m0_n, n0_n, 1);
     stage ^= 1;
 
@@ -1188,15 +1260,15 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     if (wave_stores) {
       char* slab = smem + SLABS + wave * 4096;
       if constexpr (HALF_SLABS) {
-        if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
-        else store_wave_tile_h<MB, NB, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        else store_wave_tile_h<MB, NB, QKV, false, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       } else {
         if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
         else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
       }
     }
     if (!has_next) break;
-    read_frags(stage, 0, 0);
+    read_first(stage);
     prev_stored = wave_stores;
     vp = vp_next;
     m0 = m0_n;
@@ -1310,19 +1382,34 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
                    smem_base + (unsigned)stage * STAGE + (unsigned)wave * 8192u + q * 1024);
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> 1) & 7;
-  const int a_row_off = (wm * TM + frow) * ROWB;
-  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
-  h8 af[2][MB], bf[2][NB];
-  auto read_frags = [&](int stage, int ks, int slot) __attribute__((always_inline)) {
+  // Fragments of v_mfma_f32_16x16x32_f16: a lane supplies row lane % 16 of a block of 16 rows and
+  // the 8 halves of 16-byte unit lane / 16 of a 32-wide k-step.  (Which k goes to which lane group
+  // is free as long as both operands agree: k is summed over.)  16 consecutive lanes read 16
+  // consecutive rows at one unit, as with the 32-row fragments of the small-tile kernel: no bank
+  // conflicts.
+  const int lrow = lane & 15, lq = lane >> 4, fkey = (lrow >> 1) & 7;
+  const int a_row_off = (wm * TM + lrow) * ROWB;
+  const int b_row_off = BM * ROWB + (wn * TN + lrow) * ROWB;
+  // A slice = one 32-wide k-step s times one half h of the sub-tile's rows: 4 A blocks (af; a
+  // block's register takes the next slice's block as soon as its four MFMAs are issued) times 4 B
+  // blocks (bf[s], good for both halves of step s).
+  static_assert(TM == 128 && TN == 64, "128 x 64 sub-tiles");
+  h8 af[4], bf[2][4];
+  auto frag_a = [&](const char* st, int h, int jl, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(st + a_row_off + (h * 64 + jl * 16) * ROWB +
+                                        (((s * 4 + lq) ^ fkey) << 4));
+  };
+  auto frag_b = [&](const char* st, int i, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(st + b_row_off + i * 16 * ROWB +
+                                        (((s * 4 + lq) ^ fkey) << 4));
+  };
+  // the fragments of a k-tile's first slice
+  auto read_first = [&](int stage) __attribute__((always_inline)) {
     const char* st = smem + stage * STAGE;
-    const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
-    for (int j = 0; j < MB; ++j)
-      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
+    for (int jl = 0; jl < 4; ++jl) af[jl] = frag_a(st, 0, jl, 0);
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
+    for (int i = 0; i < 4; ++i) bf[0][i] = frag_b(st, i, 0);
   };
   auto barrier_lds = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
@@ -1333,7 +1420,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
   issue(1, m0, n0, 1);
   wait_vmcnt<LPT>();
   asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
+  read_first(0);
   int stage = 0;  // stage of the k-tile being multiplied
 
   while (true) {
@@ -1347,42 +1434,44 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     // barriers, and has no residual, bias or output of its own
     const bool wave_stores = nw0 < N;
 
-    f16v acc[NB][MB];
+    // acc[i][j] = the 16 x 16 block of columns 16 i.., rows 16 j.. of the sub-tile: a lane holds
+    // row lane % 16 and the 4 columns 4 (lane / 16) + 0..3
+    f4 acc[2 * NB][2 * MB];
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
+    for (int i = 0; i < 2 * NB; ++i)
 #pragma unroll
-      for (int j = 0; j < MB; ++j)
+      for (int j = 0; j < 2 * MB; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    // One k-slice, as in gemm_stream_kernel: eight MFMAs on fragment slot `slot`, the six
-    // fragment reads of slice `rks` of `rstage` behind the first six of them, `extra(q)` behind
-    // MFMA q.
-    auto slice = [&](int slot, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+    // One slice, as in gemm_stream_kernel: eight pairs of MFMAs, the fragment reads for slice
+    // `rks` of `rstage` behind them, `extra(q)` behind pair q.
+    auto slice = [&](int, bool fetch, int rstage, int rks, auto&& extra) __attribute__((always_inline)) {
+      // this slice is t = rks - 1 (mod 4): k-step s = t / 2, row half h = t % 2
+      const int t = (rks + 3) & 3, s = t >> 1, h = t & 1;
       const char* st = smem + rstage * STAGE;
-      const int choff = ((rks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+      for (int q = 0; q < 8; ++q) {
+        const int jl = q >> 1;
 #pragma unroll
-        for (int jj = 0; jj < MB; ++jj) {
-          const int q = i * MB + jj;
-          const int j = (i & 1) ? MB - 1 - jj : jj;  // one operand changes per MFMA
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[slot][i], af[slot][j], acc[i][j],
-                                                             0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          if (fetch) {
-            if (q == 0)
-              bf[slot ^ 1][0] = *reinterpret_cast<const h8*>(st + b_row_off + choff);
-            else if (q <= MB)
-              af[slot ^ 1][q - 1] =
-                  *reinterpret_cast<const h8*>(st + a_row_off + (q - 1) * 32 * ROWB + choff);
-            else if (q < MB + NB)
-              bf[slot ^ 1][q - MB] =
-                  *reinterpret_cast<const h8*>(st + b_row_off + (q - MB) * 32 * ROWB + choff);
-          }
-          extra(q);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int p = 0; p < 2; ++p) {
+          const int ii = (q & 1) * 2 + p;
+          const int i = (jl & 1) ? 3 - ii : ii;  // one operand changes per MFMA
+          acc[i][4 * h + jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bf[s][i], af[jl],
+                                                                      acc[i][4 * h + jl], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (fetch) {
+          // behind an A block's second pair: the same block of the next slice.  Behind the first
+          // pairs: the B blocks of k-step 1 (during slice 1) or of the published k-tile's k-step 0
+          // (during slice 3); each B set is idle while it is written.
+          if (q & 1) af[jl] = frag_a(st, rks & 1, jl, rks >> 1);
+          else if (t == 1) bf[1][jl] = frag_b(st, jl, 1);
+          else if (t == 3) bf[0][jl] = frag_b(st, jl, 0);
+        }
+        extra(q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     };
     auto nothing = [](int) __attribute__((always_inline)) {};
     // The three slices in front of a k-tile's last.  `extra0` deals the second half of the
@@ -1441,17 +1530,17 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     first_slices([&](int q) __attribute__((always_inline)) {
       if ((q & 1) && wave_stores) issue_res_one(stage ^ 1, res0, 4 + q / 2);
     });
-    h4 bias_raw[NB][4];
-    // all 8 loads in flight under the last slice
-    if (wave_stores) load_bias<_Float16, NB>(ep, nw0, fhalf, bias_raw);
+    h4 bias_raw[NB][2];
+    // all 4 loads in flight under the last slice
+    if (wave_stores) load_bias16<_Float16, NB>(ep, nw0, lq, bias_raw);
     __builtin_amdgcn_sched_barrier(0);
     slice(1, false, 0, 0, nothing);
-    f4 bias_r[NB][4];
-    bias_to_f32(bias_raw, bias_r);
+    f4 bias_r[NB][2];
+    bias_to_f32_16(bias_raw, bias_r);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(bias_r[i][g]));
+      for (int g = 0; g < 2; ++g) asm volatile("" : "+v"(bias_r[i][g]));
     barrier_lds();  // every wavefront has read the last k-tile's fragments
     if (wave_stores) {
       const char* res1 = res_src(m0, n0, 1);
@@ -1489,7 +1578,7 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
     if (wave_stores) wait_vmcnt<16>();
     else wait_vmcnt<8>();
     asm volatile("s_barrier" ::: "memory");
-    read_frags(stage, 0, 0);
+    read_first(stage);
     vp = vp_next;
     m0 = m0_n;
     n0 = n0_n;
