@@ -44,10 +44,10 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
 }
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
-# HBM-side bytes of one ffn1 call from rocprofv3 --pmc FETCH_SIZE (992.4 MB after scaling by
-# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.9 MB); the counters cannot be read
+# HBM-side bytes of one ffn1 call from rocprofv3 --pmc FETCH_SIZE (983.8 MB after scaling by
+# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.7 MB); the counters cannot be read
 # from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
-FFN1_TRAFFIC_BYTES = 1.936e9
+FFN1_TRAFFIC_BYTES = 1.928e9
 
 
 def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
@@ -220,6 +220,9 @@ def main():
                     help="include the tied LM head (logits [T, 50257]) in the step")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the host-CPU leg (used under rocprofv3)")
+    ap.add_argument("--no-zero-operands", action="store_true",
+                    help="skip the ffn1 run on all-zero operands behind the timed region (used "
+                         "under rocprofv3, so that the trace holds the forward's launches only)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain copy kernel of known size (1 GiB read, 1 GiB "
                          "written) so that FETCH_SIZE / WRITE_SIZE counters of the same "
@@ -320,7 +323,7 @@ def main():
                      "avg_ms": round(ffn1_ms, 4), "calls": len(ffn1_events),
                      "traffic": FFN1_TRAFFIC_BYTES if arch is ARCH and batch == BATCH else None},
     }
-    if headline:
+    if headline and not args.no_zero_operands:
         # the same ffn1 call on all-zero operands (outside the timed region): identical
         # instructions, no bit toggling, so the clock stays up -- the rate the kernel's schedule
         # allows, beside the rate the chip sustains on real data
