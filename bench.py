@@ -3,12 +3,13 @@
 synthetic N(0, 0.02) weights and uniform token ids, one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload headline|batch2048|xl|ops] [--lm-head]
+                    [--workload headline|batch2048|xl|ops|mfma] [--lm-head]
 
 The default (and the only line the contract asks for) is `headline`; `batch2048` is the same model
 at the max-batch memory point 2048 x 300, `xl` the GPT-2 XL shape (48 x 1600, 25 heads, batch 64 x
 seqlen 1024), `ops` times the single operators at the headline sizes (mean and median of
-event-timed repetitions, one JSON line).  `--lm-head` adds the tied LM head (logits) to the step.
+event-timed repetitions, one JSON line), `mfma` what a loop of nothing but MFMAs sustains on this
+chip by instruction shape and operand data.  `--lm-head` adds the tied LM head (logits) to the step.
 
 A step is one forward pass (hidden state [512, 300, 768], like the reference's forward, which
 stops at the final LayerNorm) with the token ids already resident in HBM.  Prints ONE JSON
@@ -210,12 +211,48 @@ def bench_ops(dev):
                       "n_gpus": 1, "ops": rows}), flush=True)
 
 
+def bench_mfma(dev):
+    """What a loop of nothing but MFMAs sustains on this chip (gptmi_probe_mfma: one workgroup of
+    8 wavefronts per CU, the register footprint of a GEMM wavefront), by instruction shape, with
+    and without the GEMM kernels' LDS fragment reads, on N(0, 1) operands and on zeros."""
+    import torch
+
+    from gpt_triton_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    g = torch.Generator(device=dev).manual_seed(1337)
+    rnd = torch.randn(1 << 23, device=dev, generator=g).half()   # 16 MiB
+    zer = torch.zeros_like(rnd)
+    sink = torch.zeros(1024, device=dev)
+    ksteps = 2000  # 2000 x 2 wavefronts per SIMD x 512 cycles: ~1 ms at full rate
+    rows = []
+    for shape in (32, 16):
+        for lds in (0, 1):
+            for name, data in (("N(0,1)", rnd), ("zeros", zer)):
+                def fn():
+                    _lib.check(lib.gptmi_probe_mfma(shape, lds, data.data_ptr(), sink.data_ptr(),
+                                                    ksteps, cus,
+                                                    torch.cuda.current_stream().cuda_stream),
+                               "probe_mfma")
+                mean, med, n = time_op(fn)
+                flops = 2.0 * (1 << 18) * ksteps * 8 * cus  # 64 x 128 x 32 MACs per k-step and wavefront
+                rows.append({"mfma": "32x32x16" if shape == 32 else "16x16x32",
+                             "lds_fragment_reads": bool(lds), "operands": name,
+                             "mean_ms": round(mean, 4), "reps": n,
+                             "tflops": round(flops / (mean * 1e-3) / 1e12, 1),
+                             "frac_mfma_peak": round(flops / (mean * 1e-3) / PEAK_FP16, 4)})
+    assert not bool(sink.any())
+    print(json.dumps({"metric": "mfma_loop_sustained", "dtype": "f16", "n_gpus": 1,
+                      "workgroups": cus, "rows": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ops"], default="headline")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ops", "mfma"], default="headline")
     ap.add_argument("--lm-head", action="store_true",
                     help="include the tied LM head (logits [T, 50257]) in the step")
     ap.add_argument("--no-cpu-baseline", action="store_true",
@@ -243,6 +280,8 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "ops":
         return bench_ops(dev)
+    if args.workload == "mfma":
+        return bench_mfma(dev)
 
     arch, batch, seqlen, what = WORKLOADS[args.workload]
     headline = args.workload == "headline" and not args.lm_head

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libgptmi.so")
-SOURCES = ["rowops.hip", "gemm.hip", "flash_attn.hip", "capi.cpp"]
+SOURCES = ["rowops.hip", "gemm.hip", "flash_attn.hip", "probe.hip", "capi.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -44,7 +44,7 @@ def build(verbose=True):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.rsplit(".", 1)[0] + ".o") for s in SOURCES]
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=5) as ex:
         list(ex.map(_compile, SOURCES, objs))
     tmp = LIB_PATH + ".tmp"
     r = subprocess.run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs],

@@ -241,6 +241,20 @@ int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out,
                      float scale, float p, uint64_t seed, int olayout, int dtype,
                      void* stream);
 
+/*
+ * Matrix-pipe probe for the benchmark (no counterpart in the reference; not on the forward path).
+ * `workgroups` workgroups of 8 wavefronts (2 per SIMD when one workgroup runs per CU) each execute
+ * `ksteps` (even) 32-wide k-steps of the MFMAs of a 64 x 128 wavefront sub-tile -- 2^19 FLOP per
+ * k-step and wavefront -- with v_mfma_f32_32x32x16_f16 (shape 32) or v_mfma_f32_16x16x32_f16
+ * (shape 16), the register footprint of a GEMM wavefront, and nothing else; with lds_reads != 0
+ * the 12 operand fragments of every k-step are read from LDS between the MFMAs as the GEMM
+ * kernels do.  The operand values come from `operands` (16 MiB of fp16 on the device: what the
+ * chip sustains depends on how many bits toggle -- zeros and N(0, 1) values differ by a third);
+ * `sink` is 4 KiB of device memory that stays unwritten.  Only enqueues work on `stream`.
+ */
+int gptmi_probe_mfma(int shape, int lds_reads, const void* operands, void* sink,
+                     int64_t ksteps, int64_t workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1013,3 +1013,22 @@ def test_fused_ffn_degenerate_sizes(K, gpu_device, dtype, M, N, Kd):
     b = r.standard_normal(N).astype(NP[dtype])
     z = host(K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device)))
     check(z, O.fused_ffn(x, w, bias=b), dtype, f"ffn {M}x{N}x{Kd}")
+
+
+def test_mfma_probe_runs_and_writes_nothing(gpu_device):
+    """The benchmark's matrix-pipe probe (bench.py --workload mfma): both instruction shapes, with
+    and without LDS fragment reads, finish and leave the sink untouched."""
+    from gpt_triton_amd import _lib
+
+    lib = _lib.load()
+    data = torch.randn(1 << 23, device=gpu_device).half()
+    sink = torch.zeros(1024, device=gpu_device)
+    with torch.cuda.device(gpu_device):
+        st = torch.cuda.current_stream().cuda_stream
+        for shape in (16, 32):
+            for lds in (0, 1):
+                _lib.check(lib.gptmi_probe_mfma(shape, lds, data.data_ptr(), sink.data_ptr(), 64, 8,
+                                                st), "probe_mfma")
+        torch.cuda.synchronize()
+    assert not bool(sink.any())
+
