@@ -196,6 +196,19 @@ def bench_ops(dev):
         ("embedding 512x300x768", lambda: K.fused_embeddings(ids, wte, wpe), None, M * 8 + 2 * M * h * 2 + SEQLEN * h * 2, flush),
         ("embedding + first LayerNorm 512x300x768", lambda: K.fused_embeddings_layer_norm(ids, wte, wpe, lw, lb), None, M * 8 + 3 * M * h * 2 + SEQLEN * h * 2, flush),
     ]
+    # where the streamed operand comes from: a product whose activations (201 MB) fit the 256 MB
+    # memory-side cache, repeated with the cache left alone and with it flushed (HBM) in between,
+    # on N(0, 1) and on all-zero operands
+    Mc = 32768
+    xc, wc, bc = rn(Mc, 4 * h), K.pack_weight(rn(4 * h, 2 * h, std=0.02)), rn(2 * h, std=0.02)
+    xcz, wcz, bcz = torch.zeros_like(xc), K.pack_weight(torch.zeros(4 * h, 2 * h, device=dev).half()), torch.zeros_like(bc)
+    gc = 2 * Mc * 2 * h * 4 * h
+    ops += [
+        ("32768x3072 -> 1536 +bias, activations in the memory-side cache", lambda: K.fused_ffn(xc, wc, bias=bc), gc, None, None),
+        ("32768x3072 -> 1536 +bias, activations from HBM", lambda: K.fused_ffn(xc, wc, bias=bc), gc, None, flush),
+        ("32768x3072 -> 1536 +bias, all-zero operands, activations in the memory-side cache", lambda: K.fused_ffn(xcz, wcz, bias=bcz), gc, None, None),
+        ("32768x3072 -> 1536 +bias, all-zero operands, activations from HBM", lambda: K.fused_ffn(xcz, wcz, bias=bcz), gc, None, flush),
+    ]
     rows = []
     for name, fn, flops, nbytes, fl in ops:
         mean, med, n = time_op(fn, fl)
