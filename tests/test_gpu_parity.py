@@ -341,6 +341,35 @@ def test_fused_ffn_random_shapes(K, gpu_device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,Kd", [(2048, 320, 128),    # two k-tiles: the least the streaming kernel takes
+                                    (2048, 256, 192),    # three: the least with a residual
+                                    (8192, 2304, 128),   # 288 tiles: some workgroups walk a second tile
+                                    (8192, 2368, 192),   # the same with a column edge (N % 256 = 64)
+                                    (8192, 2304, 256)])
+def test_streaming_gemm_fewest_k_tiles_and_second_tile(K, gpu_device, dtype, M, N, Kd):
+    """The persistent kernels at the short end of their k loop (the first, middle and last k-tiles
+    are separate code) and across a tile boundary inside one workgroup; every element against the
+    fp32 product of the fp16-rounded operands, with and without GELU / residual."""
+    g = torch.Generator(device="cpu").manual_seed(M + N + Kd)
+    x = torch.randn((M, Kd), generator=g).to(dtype).to(gpu_device)
+    w = (torch.randn((Kd, N), generator=g) / Kd ** 0.5).to(dtype).to(gpu_device)
+    b = torch.randn(N, generator=g).to(dtype).to(gpu_device)
+    rs = torch.randn((M, N), generator=g).to(dtype).to(gpu_device)
+    base = x.half().float() @ w.half().float() + b.float()
+    for gelu, res in ((False, False), (True, False), (False, True), (True, True)):
+        z = K.fused_ffn(x, w, bias=b, residual=rs if res else None, add_gelu=gelu)
+        want = torch.nn.functional.gelu(base, approximate="tanh") if gelu else base
+        if res:
+            want = want + rs.float()
+        check(host(z), want.cpu().numpy(), dtype, f"{M}x{N}x{Kd} gelu={gelu} res={res}")
+    if N % 192 == 0:  # three equal parts of whole heads: the head-major scatter of the same product
+        heads = N // 192
+        q, k_, v = K.matmul_and_split_qkv(x.view(M // 128, 128, Kd), w, b, heads)
+        got = torch.cat([t.transpose(1, 2).reshape(M, N // 3) for t in (q, k_, v)], dim=1)
+        check(host(got), base.cpu().numpy(), dtype, f"qkv {M}x{N}x{Kd}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("M,N,Kd", [(300, 768, 3072),    # 18 tiles of 128 x 128: the 64 x 64 tiles
                                     (333, 200, 70),      # the same, ragged in M, N and K
                                     (768, 2304, 768),    # 108: the 64 x 128 tiles
