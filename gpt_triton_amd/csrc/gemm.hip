@@ -1678,11 +1678,12 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
   // buffered (2 x 64 KB of LDS).  Small ones: 128x128 tiles, 4 wavefronts, K step 32, 4-stage
   // ring, so that a few hundred rows still spread over several CUs.
   if (M >= 2048 && N >= 256) {
-    // Whole row tiles, N a multiple of 64 (the wavefronts of the last column tile whose 64
-    // columns lie past the edge store nothing), at least two k-tiles, vector epilogue (16-byte
-    // stores for fp16), no dropout, no residual: the streaming kernel.  It has neither row edge
-    // handling nor the generator.
-    if (M % 256 == 0 && N % 64 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
+    // N a multiple of 64 (the wavefronts of the last column tile whose 64 columns lie past the
+    // edge store nothing), at least two k-tiles, vector epilogue (16-byte stores for fp16), no
+    // dropout, no residual: the streaming kernel on the whole row tiles.  It has neither row edge
+    // handling nor the generator; rows past the last whole tile go to the small tiles below.
+    const int64_t m_full = M / 256 * 256;
+    if (N % 64 == 0 && Kp >= 128 && Kp <= (1 << 21) && ep.vec_ok &&
         (sizeof(T) == 4 || ep.vec8_ok) && !(ep.drop.p > 0.f) && ep.residual == nullptr) {
       // Every persistent workgroup walks ceil(tiles / CUs) tiles, so a few tiles beyond a whole
       // number of rounds cost a full round.  Then the last rows leave the persistent launch --
@@ -1691,9 +1692,9 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
       // tiles; 597 of the 600 row tiles stay, 768 rows follow as 288 tiles of 64 x 128).
       const int cus = cu_count();
       if (cus < 0) return cus;
-      const int64_t tiles_m = M / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
+      const int64_t tiles_m = m_full / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
       const int64_t rounds = tiles / cus, rem = tiles % cus;
-      int64_t m_head = M;
+      int64_t m_head = m_full;
       if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;
       int rc = launch_stream<2, 4, T, QKV>(A, Bt, m_head, N, Kp, ep, st);
       if (rc != 0 || m_head == M) return rc;
@@ -1707,16 +1708,16 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
     if constexpr (sizeof(T) == 2 && !QKV) {
       if (ep.residual != nullptr && !(ep.drop.p > 0.f) && ep.vec8_ok && Kp >= 128 &&
           (((uintptr_t)ep.residual) & 15) == 0) {
-        if (M % 256 == 0 && N % 64 == 0 && Kp >= 192 && Kp <= (1 << 21)) {
-          // whole row tiles, N a multiple of 64 and at least three k-tiles: the streaming
-          // kernel, with the same cut as above -- the row tiles that fill whole rounds of the
+        if (N % 64 == 0 && Kp >= 192 && Kp <= (1 << 21)) {
+          // N a multiple of 64 and at least three k-tiles: the streaming kernel on the whole row
+          // tiles, with the same cut as above -- the row tiles that fill whole rounds of the
           // persistent workgroups stay, the rest (headline N = 768: 1800 tiles = 7 rounds + 8;
           // 597 of 600 row tiles stay) go to the small tiles
           const int cus = cu_count();
           if (cus < 0) return cus;
-          const int64_t tiles_m = M / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
+          const int64_t tiles_m = m_full / 256, tiles_n = (N + 255) / 256, tiles = tiles_m * tiles_n;
           const int64_t rounds = tiles / cus, rem = tiles % cus;
-          int64_t m_head = M;
+          int64_t m_head = m_full;
           if (rounds >= 4 && rem != 0 && rem * 4 <= cus) m_head = rounds * cus / tiles_n * 256;
           int rc = launch_stream_res(A, Bt, m_head, N, Kp, ep, st);
           if (rc != 0 || m_head == M) return rc;
