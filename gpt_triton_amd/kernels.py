@@ -96,14 +96,15 @@ def pack_weight(weight):
 
 @torch.no_grad()
 def pack_lm_head(wte):
-    """Packs wte [V, H] once for `lm_head`, with the vocabulary padded to a multiple of 8 by zero
+    """Packs wte [V, H] once for `lm_head`, with the vocabulary padded to a multiple of 64 by zero
     rows.  GPT-2's V = 50257 is odd: rows of a dense [T, V] fp16 matrix then start on 2-byte
     boundaries and every logit is stored on its own.  With the padded image the GEMM writes
-    [T, Vp] rows of whole 16-byte units and `lm_head` returns the [.., :V] view of it."""
+    [T, Vp] rows of whole 128-byte lines -- the shape the persistent GEMM kernel takes -- and
+    `lm_head` returns the [.., :V] view of it."""
     assert wte.dim() == 2 and wte.is_contiguous()
     dev = _on_gpu(wte)
     V, H = wte.shape
-    Vp = -(-V // 8) * 8
+    Vp = -(-V // 64) * 64
     lib = _lib.load()
     buf = torch.zeros(lib.gptmi_packed_weight_bytes(Vp, H), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -261,7 +262,7 @@ def fused_ffn(x, weight, bias=None, residual=None, add_gelu=False, dropout_prob=
 def lm_head(x, wte):
     """x @ wte^T: logits [*, V].  `wte` is the [V, H] embedding matrix itself (read in place, no
     transposed copy; the result is contiguous) or its `pack_lm_head` image (the result is then
-    the [*, :V] view of a buffer whose rows are padded to a multiple of 8 logits)."""
+    the [*, :V] view of a buffer whose rows are padded to a multiple of 64 logits)."""
     out_shape_0 = x.shape[:-1]
     x = x.view((-1, x.shape[-1]))
     assert x.is_contiguous()

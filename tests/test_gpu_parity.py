@@ -398,16 +398,17 @@ def test_lm_head_transposed_weight(K, gpu_device, dtype):
     assert z.shape == (130, 50257)
     want = O.fused_ffn(x, np.ascontiguousarray(wte.T))
     check(host(z), want, dtype, "lm_head")
-    # the zero-padded packed image: same logits, as a view of rows padded to 50264
+    # the zero-padded packed image: same logits, as a view of rows padded to 50304 (a multiple of 64)
     image = K.pack_lm_head(dev(wte, gpu_device))
     zp = K.lm_head(dev(x, gpu_device).view(2, 65, 768), image)
-    assert zp.shape == (2, 65, 50257) and zp.stride() == (65 * 50264, 50264, 1)
+    assert zp.shape == (2, 65, 50257) and zp.stride() == (65 * 50304, 50304, 1)
     check(host(zp).reshape(130, 50257), want, dtype, "lm_head padded")
 
 
 def test_lm_head_padded_big_tiles(K, gpu_device):
-    """M = 2600 rows (the 256 x 256 kernel) x 50257 logits through the padded image; sampled
-    rows against the oracle, and the 7 padding columns of the underlying buffer are zero."""
+    """M = 2600 rows (the persistent kernel on the first 2560, the small tiles on the rest) x 50257
+    logits through the padded image; sampled rows against the oracle, and the 47 padding columns of
+    the underlying buffer are zero."""
     r = np.random.default_rng(22)
     x = r.standard_normal((2600, 768)).astype(np.float16)
     wte = (0.02 * r.standard_normal((50257, 768))).astype(np.float16)
@@ -416,7 +417,7 @@ def test_lm_head_padded_big_tiles(K, gpu_device):
     rows = [0, 255, 256, 2559, 2560, 2599]
     want = O.fused_ffn(x[rows], np.ascontiguousarray(wte.T))
     check(host(z[rows]), want, torch.float16, "lm_head padded, big tiles")
-    full = torch.as_strided(z, (2600, 50264), (50264, 1))
+    full = torch.as_strided(z, (2600, 50304), (50304, 1))
     assert (full[:, 50257:] == 0).all()
 
 
