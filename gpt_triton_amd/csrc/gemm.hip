@@ -36,9 +36,12 @@
 //     the 8 XCDs) gets a contiguous range of tiles; inside a group of column tiles whose
 //     weight panels fit the XCD's L2 the column runs fastest, so the tiles that share a row
 //     block of A run on the same L2 at the same time.
-// gemm_stream_kernel (further down) is the persistent form of the 256 x 256 x 64 configuration
-// for whole-tile shapes without residual: one workgroup per CU walks tiles and the pipeline
-// runs across tile boundaries.  launch_shape (at the end) picks kernel and configuration.
+// gemm_stream_kernel and gemm_stream_res_kernel (further down) are the persistent forms of the
+// 256 x 256 x 64 configuration for whole row tiles, without and with a residual: one workgroup
+// per CU walks tiles and the pipeline runs across tile boundaries.  They multiply with
+// v_mfma_f32_16x16x32_f16 (a sub-tile is 16 x 16 blocks there; same LDS layout, same products,
+// less power per product on operands that toggle bits, so a higher clock).  launch_shape (at the
+// end) picks kernel and configuration.
 #include "common.h"
 #include "launch.h"
 
