@@ -3,13 +3,12 @@
 synthetic N(0, 0.02) weights and uniform token ids, one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload headline|batch2048|xl|ops|mfma] [--lm-head]
+                    [--workload headline|batch2048|xl|ops] [--lm-head]
 
 The default (and the only line the contract asks for) is `headline`; `batch2048` is the same model
 at the max-batch memory point 2048 x 300, `xl` the GPT-2 XL shape (48 x 1600, 25 heads, batch 64 x
 seqlen 1024), `ops` times the single operators at the headline sizes (mean and median of
-event-timed repetitions, one JSON line), `mfma` what a loop of nothing but MFMAs sustains on this
-chip by instruction shape and operand data.  `--lm-head` adds the tied LM head (logits) to the step.
+event-timed repetitions, one JSON line).  `--lm-head` adds the tied LM head (logits) to the step.
 
 A step is one forward pass (hidden state [512, 300, 768], like the reference's forward, which
 stops at the final LayerNorm) with the token ids already resident in HBM.  Prints ONE JSON
@@ -19,8 +18,9 @@ line.  Beside the whole-forward numbers it carries
     the persistent kernel plus, at this shape, one of the small-tile kernel for the last 768
     rows); achieved = 2*M*N*K / mean duration against the 2.5 PFLOP/s dense fp16 MFMA peak;
   * "cpu_baseline": the plain PyTorch fp32 forward of the same architecture (the stand-in for the
-    reference's CPU-side comparator, HF GPT2Model in fp32) on this box's host cores, on a
-    bounded sample of the same workload.
+    reference's CPU-side comparator, HF GPT2Model in fp32) on this box's host cores, at the
+    same 512 x 300 batch (1 warm-up + 3 timed forwards, about two minutes on 16 cores;
+    `--cpu-sample-batch 64` bounds it for profile runs).
 """
 import argparse
 import json
@@ -45,10 +45,21 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
 }
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
-# HBM-side bytes of one ffn1 call from rocprofv3 --pmc FETCH_SIZE (983.8 MB after scaling by
-# the copy kernel of --traffic-calibration) + WRITE_SIZE (943.7 MB); the counters cannot be read
-# from inside this process, so the figure is the one of profiles/gemm_ffn1_hbm_traffic_pmc.md
-FFN1_TRAFFIC_BYTES = 1.928e9
+# HBM-side bytes of one ffn1 call come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (scaled
+# by the copy kernel of --traffic-calibration); the counters cannot be read from inside this
+# process, so the figure is the one the profile summary states in its `ffn1_call_hbm_bytes:` line
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_ffn1_hbm_traffic_pmc.md")
+
+
+def ffn1_traffic_bytes():
+    """The `ffn1_call_hbm_bytes: <number>` line of the traffic profile, or None without it."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("ffn1_call_hbm_bytes:"):
+                return float(line.split(":", 1)[1].split()[0])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def forward_flops(tokens, seqlen, arch=ARCH, lm_head=False):
@@ -70,9 +81,10 @@ def cpu_model_name():
     return "unknown CPU"
 
 
-def cpu_baseline(sample_batch=64, reps=3):
+def cpu_baseline(sample_batch=BATCH, reps=3):
     """PyTorch fp32 eager forward of the same 124M model on the host cores: 1 warm-up + `reps`
-    timed forwards of `sample_batch` x 300 tokens (about 15 s of CPU work on 16 cores)."""
+    timed forwards of `sample_batch` x 300 tokens (the whole 512 x 300 step by default: about
+    30 s per forward on 16 cores)."""
     import torch
 
     from oracle import gpt2_oracle as O
@@ -99,7 +111,7 @@ def cpu_baseline(sample_batch=64, reps=3):
             "cpu_tokens_per_s_best": round(tokens / best, 1),
             "sample": f"PyTorch fp32 eager forward of the same 124M model on the host CPU "
                       f"({threads} torch threads), batch {sample_batch} x seqlen {SEQLEN} "
-                      f"({tokens} tokens; the full 512 x 300 step would take ~{mean * 512 / sample_batch:.0f} s), "
+                      f"({tokens} tokens" + ("" if sample_batch == BATCH else f"; the full 512 x 300 step would take ~{mean * BATCH / sample_batch:.0f} s") + "), "
                       f"1 warm-up + {reps} timed forwards: mean {mean * 1e3:.0f} ms, min {best * 1e3:.0f} ms"}
 
 
@@ -224,52 +236,19 @@ def bench_ops(dev):
                       "n_gpus": 1, "ops": rows}), flush=True)
 
 
-def bench_mfma(dev):
-    """What a loop of nothing but MFMAs sustains on this chip (gptmi_probe_mfma: one workgroup of
-    8 wavefronts per CU, the register footprint of a GEMM wavefront), by instruction shape, with
-    and without the GEMM kernels' LDS fragment reads, on N(0, 1) operands and on zeros."""
-    import torch
-
-    from gpt_triton_amd import _lib
-
-    lib = _lib.load()
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    g = torch.Generator(device=dev).manual_seed(1337)
-    rnd = torch.randn(1 << 23, device=dev, generator=g).half()   # 16 MiB
-    zer = torch.zeros_like(rnd)
-    sink = torch.zeros(1024, device=dev)
-    ksteps = 2000  # 2000 x 2 wavefronts per SIMD x 512 cycles: ~1 ms at full rate
-    rows = []
-    for shape in (32, 16):
-        for lds in (0, 1):
-            for name, data in (("N(0,1)", rnd), ("zeros", zer)):
-                def fn():
-                    _lib.check(lib.gptmi_probe_mfma(shape, lds, data.data_ptr(), sink.data_ptr(),
-                                                    ksteps, cus,
-                                                    torch.cuda.current_stream().cuda_stream),
-                               "probe_mfma")
-                mean, med, n = time_op(fn)
-                flops = 2.0 * (1 << 18) * ksteps * 8 * cus  # 64 x 128 x 32 MACs per k-step and wavefront
-                rows.append({"mfma": "32x32x16" if shape == 32 else "16x16x32",
-                             "lds_fragment_reads": bool(lds), "operands": name,
-                             "mean_ms": round(mean, 4), "reps": n,
-                             "tflops": round(flops / (mean * 1e-3) / 1e12, 1),
-                             "frac_mfma_peak": round(flops / (mean * 1e-3) / PEAK_FP16, 4)})
-    assert not bool(sink.any())
-    print(json.dumps({"metric": "mfma_loop_sustained", "dtype": "f16", "n_gpus": 1,
-                      "workgroups": cus, "rows": rows}), flush=True)
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ops", "mfma"], default="headline")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ops"], default="headline")
     ap.add_argument("--lm-head", action="store_true",
                     help="include the tied LM head (logits [T, 50257]) in the step")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the host-CPU leg (used under rocprofv3)")
+    ap.add_argument("--cpu-sample-batch", type=int, default=BATCH,
+                    help="sequences in the host-CPU forward (default: the whole batch of 512; "
+                         "64 keeps a profile run short)")
     ap.add_argument("--no-zero-operands", action="store_true",
                     help="skip the ffn1 run on all-zero operands behind the timed region (used "
                          "under rocprofv3, so that the trace holds the forward's launches only)")
@@ -293,8 +272,6 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "ops":
         return bench_ops(dev)
-    if args.workload == "mfma":
-        return bench_mfma(dev)
 
     arch, batch, seqlen, what = WORKLOADS[args.workload]
     headline = args.workload == "headline" and not args.lm_head
@@ -319,7 +296,7 @@ def main():
 
     recording = [False]
     G.fused_ffn = timed_ffn
-    step = (lambda: model(ids, return_logits=True)[0]) if args.lm_head else (lambda: model(ids))
+    step = (lambda: model(ids, return_logits=True)) if args.lm_head else (lambda: model(ids))
 
     with torch.no_grad():
         for _ in range(args.warmup):
@@ -332,6 +309,14 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     recording[0] = False
+    if args.lm_head:
+        out, logits = out
+        assert logits.shape == (batch, seqlen, arch["vocab_size"])
+        # every logit finite, and the last token row equal to the plain product of its hidden
+        # state with wte (fp32 torch): the rows past 2^32 bytes of the logits are real results
+        assert bool(torch.isfinite(logits).all())
+        ref = out[-1, -4:].float() @ model.wte_weight.data.float().t()
+        assert float((logits[-1, -4:].float() - ref).abs().max()) <= 2e-2
     assert out.shape == (batch, seqlen, arch["n_embd"]) and bool(torch.isfinite(out).all())
 
     ms = dt / args.steps * 1e3
@@ -373,7 +358,7 @@ def main():
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP16 / 1e12,
                      "unit": "TFLOP/s", "frac": round(achieved * 1e12 / PEAK_FP16, 4),
                      "avg_ms": round(ffn1_ms, 4), "calls": len(ffn1_events),
-                     "traffic": FFN1_TRAFFIC_BYTES if arch is ARCH and batch == BATCH else None},
+                     "traffic": ffn1_traffic_bytes() if arch is ARCH and batch == BATCH else None},
     }
     if headline and not args.no_zero_operands:
         # the same ffn1 call on all-zero operands (outside the timed region): identical
@@ -387,7 +372,8 @@ def main():
             "avg_ms": round(zmean, 4), "frac": round(ffn1_flops / (zmean * 1e-3) / PEAK_FP16, 4),
             "note": "same launches on all-zero x, W, bias: the schedule's own rate; the difference "
                     "to `frac` is the clock the chip gives up on operands that toggle bits"}
-    line["cpu_baseline"] = None if (args.no_cpu_baseline or not headline) else cpu_baseline()
+    line["cpu_baseline"] = (None if (args.no_cpu_baseline or not headline)
+                            else cpu_baseline(args.cpu_sample_batch))
     if args.traffic_calibration:
         copy_calibration(dev)
     print(json.dumps(line), flush=True)

@@ -35,7 +35,6 @@ SIGNATURES = {
                                 _vp, _sz, _int, _vp]),
     "gptmi_flash_attn": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _f32,
                                 _u64, _int, _int, _vp]),
-    "gptmi_probe_mfma": (_int, [_int, _int, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lib = None

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libgptmi.so")
-SOURCES = ["rowops.hip", "gemm.hip", "flash_attn.hip", "probe.hip", "capi.cpp"]
+SOURCES = ["rowops.hip", "gemm.hip", "flash_attn.hip", "capi.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

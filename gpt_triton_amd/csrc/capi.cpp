@@ -271,23 +271,6 @@ int gptmi_softmax(const void* x, void* out, int64_t M, int64_t H, int dtype, voi
   return check_launch("softmax");
 }
 
-int gptmi_probe_mfma(int shape, int lds_reads, const void* operands, void* sink, int64_t ksteps,
-                     int64_t workgroups, void* stream) {
-  if (!operands || !sink || (shape != 16 && shape != 32) || ksteps < 2 || ksteps > (1 << 24) ||
-      (ksteps & 1) || workgroups < 1 || workgroups > 65536) {
-    set_error("probe_mfma: invalid argument (shape 16 or 32, an even number of k-steps up to 2^24, "
-              "1..65536 workgroups)");
-    return GPTMI_ERR_INVALID;
-  }
-  if (((uintptr_t)operands & 15) != 0) {
-    set_error("probe_mfma: operands must be 16-byte aligned");
-    return GPTMI_ERR_INVALID;
-  }
-  launch_mfma_probe(shape, lds_reads != 0, operands, sink, (int)ksteps, (int)workgroups,
-                    (hipStream_t)stream);
-  return check_launch("probe_mfma");
-}
-
 size_t gptmi_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int wlayout) {
   if (M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype)) return 0;
   return plan_linear(M, N, K, dtype, wlayout).total;

@@ -54,9 +54,4 @@ int launch_flash_attn(const void* q, const void* k, const void* v, void* out,
                       int64_t B, int64_t N, int64_t L, int64_t Lk, int d, float scale,
                       Dropout drop, bool out_blnd, bool f16, hipStream_t st);
 
-// Matrix-pipe probe (probe.hip): `workgroups` workgroups of 8 wavefronts each run `ksteps`
-// 32-wide k-steps of a 64 x 128 sub-tile's MFMAs on 16 MiB of fp16 `operands`; writes nothing.
-int launch_mfma_probe(int shape, bool lds_reads, const void* operands, void* sink, int ksteps,
-                      int workgroups, hipStream_t st);
-
 }  // namespace gptmi

@@ -186,10 +186,12 @@ class FusedGPT(nn.Module):
         return super().train(mode)
 
     def _lm_head_weight(self):
-        # A vocabulary that is not a multiple of 8 (GPT-2's 50257) gets a zero-padded packed image
-        # in eval mode, so that the logits' rows are whole 16-byte units; see kernels.pack_lm_head.
+        # In eval mode the LM head multiplies with a packed image of wte whose vocabulary is
+        # zero-padded to a multiple of 64 (GPT-2's 50257 -> 50304): the logits' rows are then
+        # whole 128-byte lines and the product runs on the persistent GEMM kernel, and the image
+        # is built once instead of on every call; see kernels.pack_lm_head.
         w = self.wte_weight
-        if self.training or w.shape[0] % 8 == 0:
+        if self.training:
             return w.data
         return self._packed.get("lm_head", w, pack_lm_head)
 
@@ -197,7 +199,9 @@ class FusedGPT(nn.Module):
         # causal by construction; no attention or padding mask is taken
         p = self.config.dropout if self.training else 0.0
         if p == 0.0 and len(self.blocks) > 0:
-            # eval mode: the first block's LayerNorm comes out of the embedding kernel
+            # eval mode: the first block's LayerNorm comes out of the embedding kernel.  The two
+            # modules of blocks[0] are called one by one, so forward hooks registered on that
+            # nn.Sequential container itself do not fire (hooks on its two modules do).
             first = self.blocks[0]
             x, y = fused_embeddings_layer_norm(x, self.wte_weight.data, self.wpe_weight.data,
                                                first[0].layer_norm_weight.data,

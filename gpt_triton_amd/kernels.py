@@ -21,6 +21,7 @@ for the embedding, the flat index m*N + n for fused_ffn, query*Lk + key for the 
 weights (kernels.py:31-34, 65-70, 245-251, 457-460).
 """
 import math
+import os
 
 import torch
 
@@ -114,6 +115,21 @@ def pack_lm_head(wte):
     return PackedWeight(buf, (H, Vp), wte.dtype, vocab=V)
 
 
+def check_token_ids(x, vocab_size):
+    """Raises IndexError if a token id lies outside [0, vocab_size).  The embedding kernels
+    themselves read no memory for such an id and use a zero wte row (the reference reads out of
+    bounds); this check costs a device synchronisation, so the operators run it only when the
+    environment variable GPTMI_CHECK_IDS is set to 1."""
+    lo, hi = int(x.min()), int(x.max())
+    if lo < 0 or hi >= vocab_size:
+        raise IndexError(f"token ids span [{lo}, {hi}] but the vocabulary has {vocab_size} rows")
+
+
+def _maybe_check_ids(x, vocab_size):
+    if os.environ.get("GPTMI_CHECK_IDS") == "1" and x.numel() > 0:
+        check_token_ids(x, vocab_size)
+
+
 def _wlayout(weight, default):
     return _lib.GPTMI_W_PACKED if isinstance(weight, PackedWeight) else default
 
@@ -133,6 +149,7 @@ def fused_embeddings(x, wte, wpe, dropout_prob=0.0):
     if wte.dtype != wpe.dtype:
         raise TypeError("fused_embeddings: wte and wpe must share a dtype")
     dev = _on_gpu(x, wte, wpe)
+    _maybe_check_ids(x, V)
     z = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     lib = _lib.load()
     with torch.cuda.device(dev):
@@ -164,6 +181,7 @@ def fused_embeddings_layer_norm(x, wte, wpe, weight, bias):
     if not (wte.dtype == wpe.dtype == weight.dtype == bias.dtype):
         raise TypeError("fused_embeddings_layer_norm: wte, wpe, weight and bias must share a dtype")
     dev = _on_gpu(x, wte, wpe, weight, bias)
+    _maybe_check_ids(x, V)
     emb = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     out = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     lib = _lib.load()

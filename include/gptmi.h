@@ -11,8 +11,14 @@
  *     point tensors of that call (activations, weights and outputs alike);
  *   - the return value is 0 on success or a negative gptmi_status; the text of
  *     the most recent failure on the calling thread is gptmi_last_error();
- *   - the library holds no mutable global state besides that thread-local
- *     message, so calls from several host threads / streams are independent.
+ *   - besides that thread-local message the library keeps, per process, only
+ *     facts it looks up once and never changes: the compute-unit count of the
+ *     device that made the first GEMM / attention call (all devices of a
+ *     process are assumed to be the same model), "kernel attribute set" flags,
+ *     and the per-device address of gptmi_linear_static's scratch array.  A
+ *     race on any of them only repeats the lookup, so calls from several host
+ *     threads / streams are independent (gptmi_linear_static excepted: see
+ *     its comment).
  *
  * Each declaration cites the reference interface it stands in for
  * (thevasudevgupta/gpt-triton, file:line).  The reference has no FFI of its
@@ -240,20 +246,6 @@ int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out,
                      int64_t B, int64_t N, int64_t Lq, int64_t Lk, int64_t d,
                      float scale, float p, uint64_t seed, int olayout, int dtype,
                      void* stream);
-
-/*
- * Matrix-pipe probe for the benchmark (no counterpart in the reference; not on the forward path).
- * `workgroups` workgroups of 8 wavefronts (2 per SIMD when one workgroup runs per CU) each execute
- * `ksteps` (even) 32-wide k-steps of the MFMAs of a 64 x 128 wavefront sub-tile -- 2^19 FLOP per
- * k-step and wavefront -- with v_mfma_f32_32x32x16_f16 (shape 32) or v_mfma_f32_16x16x32_f16
- * (shape 16), the register footprint of a GEMM wavefront, and nothing else; with lds_reads != 0
- * the 12 operand fragments of every k-step are read from LDS between the MFMAs as the GEMM
- * kernels do.  The operand values come from `operands` (16 MiB of fp16 on the device: what the
- * chip sustains depends on how many bits toggle -- zeros and N(0, 1) values differ by a third);
- * `sink` is 4 KiB of device memory that stays unwritten.  Only enqueues work on `stream`.
- */
-int gptmi_probe_mfma(int shape, int lds_reads, const void* operands, void* sink,
-                     int64_t ksteps, int64_t workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -254,3 +254,48 @@ def test_xl_forward_sampled_sequences(gpu_device):
     print(f"xl forward: max|diff| {diff.max():.4e}, median {np.median(diff):.3e}, "
           f"max|ref| {np.abs(want).max():.3f}", flush=True)
     assert diff.max() <= 2e-2
+
+
+def test_headline_logits_every_element(K, gpu_device):
+    """Benchmark configurations 0 / 3 ask for logits: the tied LM head at the headline's M = 153600
+    rows, hidden states [153600, 768] against wte [50257, 768] through the padded image
+    (kernels.pack_lm_head, gpt.py:159-161, 172-179 in the reference).  The padded output is
+    153600 x 50304 fp16 = 15.45 GB: element and byte offsets pass 2^31 and 2^32.  The buffer is
+    pre-filled with NaN; every logit is compared with the fp32 torch product computed in row
+    chunks, the 47 padding columns of every row must be zero, and the rows that hold byte 2^31,
+    byte 2^32, element 2^31 and element 2^32 of the padded buffer (with their neighbours), the
+    first rows, both sides of the seam between the persistent launch and the small-tile launch
+    (152831 | 152832) and the last row are compared with the oracle."""
+    V, H, Vp = 50257, 768, 50304
+    g = torch.Generator(device=gpu_device).manual_seed(41)
+    x = torch.randn((M_HEAD, H), generator=g, device=gpu_device).half()
+    wte = (0.02 * torch.randn((V, H), generator=g, device=gpu_device)).half()
+    image = K.pack_lm_head(wte)
+    buf = torch.full((M_HEAD, Vp), float("nan"), device=gpu_device, dtype=torch.float16)
+    print("every element: logits [153600, 50257] through the padded image", flush=True)
+    K._linear(x, image, None, None, buf, False, 0.0, K._lib.GPTMI_W_PACKED, "lm_head")
+    torch.cuda.synchronize()
+    wt = wte.float().t().contiguous()
+    n_nan = n_bad = n_pad = 0
+    scale = 0.0
+    for r0 in range(0, M_HEAD, 4096):
+        got = buf[r0:r0 + 4096]
+        want = x[r0:r0 + 4096].float() @ wt
+        gl = got[:, :V].float()
+        n_nan += int(torch.isnan(got).sum())
+        n_pad += int((got[:, V:] != 0).sum())
+        scale = max(scale, float(want.abs().max()))
+        # |b| * 2^-10 (fp16 rounding, with slack for the ordering of the fp32 sums) + a floor
+        n_bad += int(((gl - want).abs() > want.abs() * 2.0**-10 + 2.0**-12 * 4.0).sum())
+        del got, want, gl
+    assert n_nan == 0, f"{n_nan} elements were never written (NaN poison left)"
+    assert n_pad == 0, f"{n_pad} padding columns are not zero"
+    assert n_bad == 0, f"{n_bad} logits out of tolerance (max|logit| {scale:.3f})"
+    row_of = lambda off: off // Vp
+    marks = [row_of(2**31 // 2), row_of(2**32 // 2), row_of(2**31), row_of(2**32)]
+    rows = sorted({0, 1, 152831, 152832, M_HEAD - 1, *[m + d for m in marks for d in (-1, 0, 1)]})
+    assert rows[-1] == M_HEAD - 1 and 85380 in rows and 21345 in rows
+    idx = torch.tensor(rows, device=gpu_device)
+    want = O.fused_ffn(x[idx].cpu().numpy(), np.ascontiguousarray(wte.cpu().numpy().T))
+    got = buf[idx][:, :V].cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= 2 * 2.0**-10 * np.abs(want).max()

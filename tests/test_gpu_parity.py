@@ -154,6 +154,27 @@ def test_fused_embeddings_out_of_range_ids_read_nothing(K, gpu_device):
         assert np.array_equal(host(z), want)
 
 
+def test_fused_embeddings_id_check_is_opt_in(K, gpu_device, monkeypatch):
+    """GPTMI_CHECK_IDS=1 turns an id outside [0, V) into an IndexError in both embedding
+    operators; without it (the default) the call succeeds, as the test above shows."""
+    V, H, P = 50, 64, 16
+    ids = dev(np.array([[1, 2, V, 3]], dtype=np.int64), gpu_device)
+    good = dev(np.array([[1, 2, V - 1, 0]], dtype=np.int64), gpu_device)
+    wte = torch.zeros((V, H), device=gpu_device)
+    wpe = torch.zeros((P, H), device=gpu_device)
+    lw, lb = torch.ones(H, device=gpu_device), torch.zeros(H, device=gpu_device)
+    K.check_token_ids(good, V)
+    with pytest.raises(IndexError):
+        K.check_token_ids(ids, V)
+    K.fused_embeddings(ids, wte, wpe)
+    monkeypatch.setenv("GPTMI_CHECK_IDS", "1")
+    K.fused_embeddings(good, wte, wpe)
+    with pytest.raises(IndexError):
+        K.fused_embeddings(ids, wte, wpe)
+    with pytest.raises(IndexError):
+        K.fused_embeddings_layer_norm(ids, wte, wpe, lw, lb)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("H", [768, 1600, 256, 33, 4096])
 def test_fused_embeddings_layer_norm_equals_the_two_calls(K, gpu_device, dtype, H):
@@ -1043,22 +1064,3 @@ def test_fused_ffn_degenerate_sizes(K, gpu_device, dtype, M, N, Kd):
     b = r.standard_normal(N).astype(NP[dtype])
     z = host(K.fused_ffn(dev(x, gpu_device), dev(w, gpu_device), bias=dev(b, gpu_device)))
     check(z, O.fused_ffn(x, w, bias=b), dtype, f"ffn {M}x{N}x{Kd}")
-
-
-def test_mfma_probe_runs_and_writes_nothing(gpu_device):
-    """The benchmark's matrix-pipe probe (bench.py --workload mfma): both instruction shapes, with
-    and without LDS fragment reads, finish and leave the sink untouched."""
-    from gpt_triton_amd import _lib
-
-    lib = _lib.load()
-    data = torch.randn(1 << 23, device=gpu_device).half()
-    sink = torch.zeros(1024, device=gpu_device)
-    with torch.cuda.device(gpu_device):
-        st = torch.cuda.current_stream().cuda_stream
-        for shape in (16, 32):
-            for lds in (0, 1):
-                _lib.check(lib.gptmi_probe_mfma(shape, lds, data.data_ptr(), sink.data_ptr(), 64, 8,
-                                                st), "probe_mfma")
-        torch.cuda.synchronize()
-    assert not bool(sink.any())
-

@@ -69,11 +69,6 @@ def test_invalid_arguments_are_rejected_before_any_launch(lib):
                                 None, 0, 1, None) == -2                    # N = 3 * 2^26
     assert lib.gptmi_linear(fake, fake, None, None, fake, 4, 4, 4, 0, 0.0, 0, 0, None, 0, 1,
                             None) == -3                                                 # workspace
-    # the matrix-pipe probe of the benchmark: shapes 16 and 32, an even number of k-steps
-    assert lib.gptmi_probe_mfma(16, 0, None, fake, 2, 1, None) == -1
-    assert lib.gptmi_probe_mfma(8, 0, fake, fake, 2, 1, None) == -1
-    assert lib.gptmi_probe_mfma(32, 1, fake, fake, 3, 1, None) == -1
-    assert lib.gptmi_probe_mfma(32, 1, fake, fake, 2, 0, None) == -1
 
 
 def test_workspace_sizes(lib):

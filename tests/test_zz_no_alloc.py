@@ -70,3 +70,44 @@ def test_linear_static_refuses_what_does_not_fit(gpu_device):
     rc = lib.gptmi_linear_static(fake, fake, None, None, fake, 1024, 6400, 1600, 0, 0.0, 1337,
                                  _lib.GPTMI_W_KN, _lib.GPTMI_F16, None)
     assert rc == -3 and b"scratch" in lib.gptmi_last_error()
+
+
+def test_linear_static_under_graph_capture(gpu_device):
+    """What the entry point is for: after one eager call (which resolves the scratch array's
+    address on this device) it runs inside a stream capture, where an allocation or a
+    synchronisation would fail the capture; three replays with eager work between them each
+    reproduce gptmi_linear bit for bit, and the device's free memory is the same before and after
+    an eager call."""
+    lib = _lib.load()
+    dtype = torch.float16
+    pr = _problem(700, 768, 200, dtype, gpu_device, seed=21, bias=True, residual=True)
+    want = _run(lib, pr, dtype, gelu=True, static=False)
+    assert torch.equal(_run(lib, pr, dtype, gelu=True, static=True), want)
+    free0 = torch.cuda.mem_get_info(gpu_device)[0]
+    out = torch.full((pr["M"], pr["N"]), float("nan"), dtype=dtype, device=gpu_device)
+
+    def call():
+        rc = lib.gptmi_linear_static(pr["x"].data_ptr(), pr["w"].data_ptr(),
+                                     pr["bias"].data_ptr(), pr["res"].data_ptr(), out.data_ptr(),
+                                     pr["M"], pr["N"], pr["K"], 1, 0.0, 1337, _lib.GPTMI_W_KN,
+                                     CODE[dtype], torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "linear_static")
+
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(gpu_device)[0] == free0
+    side = torch.cuda.Stream(device=gpu_device)
+    side.wait_stream(torch.cuda.current_stream(gpu_device))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call()
+    torch.cuda.current_stream(gpu_device).wait_stream(side)
+    for i in range(3):
+        out.fill_(float("nan"))
+        other = pr["x"].float().sum()  # eager work and a synchronisation between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(other)
+        assert torch.equal(out, want), f"replay {i}"
