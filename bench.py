@@ -221,6 +221,30 @@ def bench_ops(dev):
         ("32768x3072 -> 1536 +bias, all-zero operands, activations in the memory-side cache", lambda: K.fused_ffn(xcz, wcz, bias=bcz), gc, None, None),
         ("32768x3072 -> 1536 +bias, all-zero operands, activations from HBM", lambda: K.fused_ffn(xcz, wcz, bias=bcz), gc, None, flush),
     ]
+    # the MLP (ffn1 + GELU -> ffn2 + residual) in one piece and in row chunks whose 3072-wide
+    # intermediate (134 / 267 MB) could stay in the 256 MB memory-side cache between the two
+    # products; 85 row tiles fill whole rounds of the persistent kernels (1020 and 255 tiles)
+    mid = torch.empty(M, 4 * h, device=dev, dtype=torch.float16)
+    mlp_out = torch.empty(M, h, device=dev, dtype=torch.float16)
+
+    def mlp(rows):
+        for r0 in range(0, M, rows):
+            r1 = min(M, r0 + rows)
+            K._linear(x[r0:r1], w1, b1, None, mid[r0:r1], True, 0.0, K._lib.GPTMI_W_PACKED, "ffn1")
+            K._linear(mid[r0:r1], w2, b2, x[r0:r1], mlp_out[r0:r1], False, 0.0,
+                      K._lib.GPTMI_W_PACKED, "ffn2")
+
+    for tiles in (600, 85, 170):
+        ops.append((f"MLP ffn1+GELU -> ffn2+residual in row chunks of {tiles} x 256 rows",
+                    (lambda t: lambda: mlp(t * 256))(tiles), gemm(3072, 768) + gemm(768, 3072), None, flush))
+    # the other head sizes the reference accepts (kernels.py:490), same number of (batch, head)
+    # pairs x head size as the headline so that the rows compare: 128 -> 6 heads, 256 -> 3 heads
+    for d, heads in ((128, 6), (256, 3)):
+        for Bq, Lq in ((BATCH, SEQLEN), (64, 1024)):
+            qa, ka, va = (rn(Bq, heads, Lq, d) for _ in range(3))
+            ops.append((f"flash attention {Bq}x{heads}x{Lq}x{d} causal",
+                        (lambda a, b, c: lambda: K.flash_attention_v1(a, b, c))(qa, ka, va),
+                        4 * Bq * heads * d * Lq * (Lq + 1) // 2, 4 * Bq * heads * Lq * d * 2, flush))
     rows = []
     for name, fn, flops, nbytes, fl in ops:
         mean, med, n = time_op(fn, fl)

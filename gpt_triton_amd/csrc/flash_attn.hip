@@ -145,8 +145,11 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   }
   // Two register sets: tile u travels in set u % 2.  It is requested two steps before it is
   // multiplied (during step u - 2) and written to LDS at the end of step u - 1, so a global load
-  // has a whole step of arithmetic plus a barrier to arrive, not a fraction of one.
-  h8 stg[2][NLD];
+  // has a whole step of arithmetic plus a barrier to arrive, not a fraction of one.  Head size
+  // 256 has room for one set only (a set is 64 registers there, beside 128 of O^T and 64 of Q):
+  // its tile u is requested at the start of step u - 1 and written at that step's end.
+  constexpr bool ONESET = D >= 256;
+  h8 stg[ONESET ? 1 : 2][NLD];
 
   auto load_tile = [&](int t, h8 (&dst)[NLD]) {
     const int k0 = t * BKEY;
@@ -194,7 +197,9 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   float mrun = -INFINITY, den = 0.f;
 
   load_tile(0, stg[0]);
-  if (nt > 1) load_tile(1, stg[1]);
+  if constexpr (!ONESET) {
+    if (nt > 1) load_tile(1, stg[1]);
+  }
   store_tile(0, stg[0]);
   __syncthreads();
 
@@ -202,7 +207,11 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   // set of tile t + 1 (written to LDS at the end) and of tile t + 2 (requested at the start,
   // into the set tile t just left) are compile-time choices
   auto step = [&](int t, h8 (&set_same)[NLD], h8 (&set_next)[NLD]) {
-    if (t + 2 < nt) load_tile(t + 2, set_same);
+    if constexpr (ONESET) {
+      if (t + 1 < nt) load_tile(t + 1, set_next);
+    } else {
+      if (t + 2 < nt) load_tile(t + 2, set_same);
+    }
     const int k0 = t * BKEY;
     if (wave_active && k0 <= qw0 + 31) {
       const char* ks_ = smem + (t & 1) * STAGE;
@@ -325,8 +334,8 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     __syncthreads();
   };
   for (int t = 0; t < nt; t += 2) {
-    step(t, stg[0], stg[1]);
-    if (t + 1 < nt) step(t + 1, stg[1], stg[0]);
+    step(t, stg[0], stg[ONESET ? 0 : 1]);
+    if (t + 1 < nt) step(t + 1, stg[ONESET ? 0 : 1], stg[0]);
   }
 
   // ---- out[q][d] = O^T[d][q] / den ------------------------------------------
