@@ -42,6 +42,8 @@
 // v_mfma_f32_16x16x32_f16 (a sub-tile is 16 x 16 blocks there; same LDS layout, same products,
 // less power per product on operands that toggle bits, so a higher clock).  launch_shape (at the
 // end) picks kernel and configuration.
+#include <stdlib.h>
+
 #include "common.h"
 #include "launch.h"
 
@@ -1589,7 +1591,10 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_res_kernel(
 }
 
 // CUs of the current device rounded down to a multiple of 8 (workgroup id % 8 = XCD for every
-// tile of a persistent launch), or a negative error code.
+// tile of a persistent launch), or a negative error code.  The environment variable
+// GPTMI_MAX_WORKGROUPS (read once) caps the number: a measurement knob -- with fewer persistent
+// workgroups than CUs the chip's power management holds a higher clock, which is how one tells a
+// kernel that is bound by the power budget from one that is bound by its own schedule.
 inline int cu_count() {
   static int num_cus = 0;  // idempotent one-time setup; a race only repeats it
   if (num_cus == 0) {
@@ -1599,6 +1604,10 @@ inline int cu_count() {
         cus < 8) {
       set_error("gemm: cannot query the CU count");
       return -4;
+    }
+    if (const char* cap = getenv("GPTMI_MAX_WORKGROUPS")) {
+      const int c = atoi(cap);
+      if (c >= 8 && c < cus) cus = c;
     }
     num_cus = cus - cus % 8;
   }

@@ -730,13 +730,20 @@ def test_forward_captured_in_a_graph(gpu_device, dtype):
         assert torch.equal(hidden, want_h) and torch.equal(logits, want_l)
 
 
-def test_gpt2_layerwise_fp32(K, gpu_device):
-    """Every operator of a 3-layer model, each fed the ORACLE's intermediate activations, so
-    that no upstream difference is carried along: fp32 storage, tolerance 1e-5 * max|b| (the
-    target for this build is 1e-4), attention through check_attention."""
-    cfg = dict(n_layer=3, n_head=4, n_embd=256, vocab_size=1000, block_size=128)
-    P = O.synthetic_params(**cfg, seed=3, std=0.05, dtype=np.float32)
-    ids = O.synthetic_ids(3, 100, cfg["vocab_size"], seed=3)
+@pytest.mark.parametrize("cfg,batch,seqlen,std", [
+    (dict(n_layer=3, n_head=4, n_embd=256, vocab_size=1000, block_size=128), 3, 100, 0.05),
+    # benchmark configuration 0: the 124M architecture, fp32, 2 x 64 tokens
+    (dict(n_layer=12, n_head=12, n_embd=768, vocab_size=50257, block_size=1024), 2, 64, 0.02),
+])
+def test_gpt2_layerwise_fp32(K, gpu_device, cfg, batch, seqlen, std):
+    """Every operator of the model, each fed the ORACLE's intermediate activations, so that no
+    upstream difference is carried along: fp32 storage, tolerance 1e-5 * max|b| (the target for
+    this build is 1e-4), attention through check_attention.  This is the tight end-to-end check
+    of the fp32 path: the chained forward (check_model_fp32) has to allow for fp16 operand
+    roundings that flip downstream of a last-bit difference."""
+    heads = cfg["n_head"]
+    P = O.synthetic_params(**cfg, seed=3, std=std, dtype=np.float32)
+    ids = O.synthetic_ids(batch, seqlen, cfg["vocab_size"], seed=3)
     D = lambda a: dev(a, gpu_device)
 
     def tight(got, want, what):
@@ -750,9 +757,9 @@ def test_gpt2_layerwise_fp32(K, gpu_device):
         y = O.fused_layer_norm(x, P[a + "layer_norm_weight"], P[a + "layer_norm_bias"])
         tight(K.fused_layer_norm(D(x), D(P[a + "layer_norm_weight"]), D(P[a + "layer_norm_bias"])),
               y, f"layer {i} ln_1")
-        q, k, v = O.matmul_and_split_qkv(y, P[a + "c_attn_weight"], P[a + "c_attn_bias"], 4)
+        q, k, v = O.matmul_and_split_qkv(y, P[a + "c_attn_weight"], P[a + "c_attn_bias"], heads)
         gq, gk, gv = K.matmul_and_split_qkv(D(y), D(P[a + "c_attn_weight"]),
-                                            D(P[a + "c_attn_bias"]), 4)
+                                            D(P[a + "c_attn_bias"]), heads)
         for g_, w_ in ((gq, q), (gk, k), (gv, v)):
             tight(g_, w_, f"layer {i} qkv")
         o = O.flash_attention_v1(q, k, v)
