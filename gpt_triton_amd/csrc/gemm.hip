@@ -1264,12 +1264,17 @@ __global__ __launch_bounds__(512, 2) void gemm_stream_kernel(
     // ---- epilogue: the next tile's first two k-tiles are landing meanwhile ----
     if (wave_stores) {
       char* slab = smem + SLABS + wave * 4096;
+      // The lane id the epilogue derives its addresses from is re-made here from a value the
+      // compiler cannot see through: otherwise it computes those addresses once, in front of the
+      // tile loop, and they occupy registers through all the k-tiles.
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
       if constexpr (HALF_SLABS) {
-        if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
-        else store_wave_tile_h<MB, NB, QKV, false, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        if (ep.gelu) store_wave_tile_h<MB, NB, QKV, true, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane_e);
+        else store_wave_tile_h<MB, NB, QKV, false, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane_e);
       } else {
-        if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
-        else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane);
+        if (ep.gelu) store_wave_tile32<MB, NB, T, QKV, true>(acc, bias_r, ep, mw0, nw0, N, slab, lane_e);
+        else store_wave_tile32<MB, NB, T, QKV, false>(acc, bias_r, ep, mw0, nw0, N, slab, lane_e);
       }
     }
     if (!has_next) break;
