@@ -276,6 +276,11 @@ def main():
     ap.add_argument("--no-zero-operands", action="store_true",
                     help="skip the ffn1 run on all-zero operands behind the timed region (used "
                          "under rocprofv3, so that the trace holds the forward's launches only)")
+    ap.add_argument("--ablate-layernorm", action="store_true",
+                    help="timing experiment, WRONG results: the 24 LayerNorm kernels between the "
+                         "GEMMs are skipped (identity), which bounds what fusing them into "
+                         "neighbouring kernels could return; prints an ablation line, not the "
+                         "benchmark line")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain copy kernel of known size (1 GiB read, 1 GiB "
                          "written) so that FETCH_SIZE / WRITE_SIZE counters of the same "
@@ -320,6 +325,15 @@ def main():
 
     recording = [False]
     G.fused_ffn = timed_ffn
+    if args.ablate_layernorm:
+        final_ln, calls = G.fused_layer_norm, [0]
+
+        def skipped_ln(x, weight, bias):
+            # the model's last call (the final LayerNorm, its output) stays; the others vanish
+            calls[0] += 1
+            return final_ln(x, weight, bias) if calls[0] % (2 * arch["n_layer"]) == 0 else x
+
+        G.fused_layer_norm = skipped_ln
     step = (lambda: model(ids, return_logits=True)) if args.lm_head else (lambda: model(ids))
 
     with torch.no_grad():
@@ -333,6 +347,12 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     recording[0] = False
+    if args.ablate_layernorm:
+        print(json.dumps({"metric": "ablation_forward_ms_with_the_layernorms_between_gemms_skipped",
+                          "value": round(dt / args.steps * 1e3, 3), "unit": "ms",
+                          "results": "wrong (timing only)", "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "config": {"workload": what}}), flush=True)
+        return
     if args.lm_head:
         out, logits = out
         assert logits.shape == (batch, seqlen, arch["vocab_size"])
