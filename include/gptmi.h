@@ -18,7 +18,10 @@
  *     and the per-device address of gptmi_linear_static's scratch array.  A
  *     race on any of them only repeats the lookup, so calls from several host
  *     threads / streams are independent (gptmi_linear_static excepted: see
- *     its comment).
+ *     its comment);
+ *   - one environment variable is read, once: GPTMI_MAX_WORKGROUPS=<n> caps
+ *     the persistent GEMM launches at n workgroups instead of one per compute
+ *     unit (a measurement knob; unset in normal use).
  *
  * Each declaration cites the reference interface it stands in for
  * (thevasudevgupta/gpt-triton, file:line).  The reference has no FFI of its
