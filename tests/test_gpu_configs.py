@@ -256,6 +256,39 @@ def test_xl_forward_sampled_sequences(gpu_device):
     assert diff.max() <= 2e-2
 
 
+@pytest.mark.parametrize("name,cfg,B,L", [
+    ("gpt2-medium", dict(n_layer=24, n_head=16, n_embd=1024, vocab_size=50257, block_size=1024), 24, 300),
+    ("gpt2-large", dict(n_layer=36, n_head=20, n_embd=1280, vocab_size=50257, block_size=1024), 16, 512),
+])
+def test_other_gpt2_sizes_forward_sampled_sequences(gpu_device, name, cfg, B, L):
+    """The GPT-2 sizes between 124M and XL that the reference's converter loads just the same
+    (gpt.py:199-247): 355M (24 x 1024, 16 heads) and 774M (36 x 1280, 20 heads), fp16, enough rows
+    for the persistent GEMM kernels with their small-tile tails (7200 / 8192 rows; 1280 and 3840
+    are 5 and 15 column tiles, 5120 is 20) and, at L = 512, the long-sequence attention kernel.
+    Hidden state and logits of two sampled sequences against the oracle, 2e-2 absolute."""
+    from gpt_triton_amd.gpt import FusedGPT, GPTConfig
+
+    params = O.synthetic_params(**cfg, seed=6, dtype=np.float16)
+    ids = O.synthetic_ids(B, L, cfg["vocab_size"], seed=6)
+    model = FusedGPT(GPTConfig(dropout=0.1, **cfg))
+    model.load_state_dict({k: torch.from_numpy(v) for k, v in params.items()})
+    model = model.to(device=gpu_device, dtype=torch.float16).eval()
+    print(f"forward {name} {B} x {L}", flush=True)
+    hidden, logits = model(torch.from_numpy(ids).to(gpu_device), return_logits=True)
+    assert hidden.shape == (B, L, cfg["n_embd"]) and bool(torch.isfinite(hidden).all())
+    assert logits.shape == (B, L, cfg["vocab_size"]) and bool(torch.isfinite(logits).all())
+    seqs = [0, B - 1]
+    idx = torch.tensor(seqs, device=gpu_device)
+    got_h = hidden[idx].cpu().numpy().astype(np.float64)
+    got_l = logits[idx].cpu().numpy().astype(np.float64)
+    del model, hidden, logits
+    torch.cuda.empty_cache()
+    want_h, want_l = O.gpt2_forward(params, ids[seqs], cfg["n_head"], lm_head=True)
+    dh, dl = np.abs(got_h - want_h).max(), np.abs(got_l - want_l).max()
+    print(f"{name}: hidden max|diff| {dh:.3e}, logits max|diff| {dl:.3e}", flush=True)
+    assert dh <= 2e-2 and dl <= 2e-2
+
+
 def test_headline_logits_every_element(K, gpu_device):
     """Benchmark configurations 0 / 3 ask for logits: the tied LM head at the headline's M = 153600
     rows, hidden states [153600, 768] against wte [50257, 768] through the padded image
