@@ -1227,6 +1227,233 @@ __global__ __launch_bounds__(256, 2) void flash_attn_ring_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Head sizes 128 and 256 in fp16 storage, equal query and key lengths, no dropout.  One
+// workgroup = 4 wavefronts = one (batch, head) x 128 queries, as in the tiled kernel, but the
+// 64-key tiles of K and V travel by direct global->LDS loads into two stages (K tile [64][D],
+// then V tile [64][D], both row-major, the swizzles applied on the source side), V is read with
+// the transposing LDS load, and no register holds a tile on its way: what the tiled kernel
+// spends on staging and on the index arrays of its staging (96 registers at head size 256,
+// which it spills) is free for O^T (D / 2 registers), Q (D / 4) and the fragments.  Head size 128
+// runs two workgroups per CU (64 KB of LDS each), head size 256 one (128 KB; a wavefront may
+// then use all 512 registers of its SIMD lane).
+//
+// LDS layout of a stage.  K row r, 16-byte unit u sits at position u ^ (r & 15): the 16 lanes
+// that read one unit of 16 consecutive rows (rows alias bank-wise, a row is 256 or 512 bytes)
+// touch 16 different bank groups.  V row r, unit u sits at position u ^ (4 (r & 3)): a
+// transposing read takes 64 contiguous bytes from each of rows r0 .. r0 + 3 (lanes 0-31) and
+// r0 + 4 .. r0 + 7 (lanes 32-63), and the swizzle puts the four rows of a half in four different
+// quarters of the banks.  Tile t + 1 is requested when the arithmetic of tile t starts (the
+// barrier in front says everyone is done with tile t - 1, whose stage it takes) and awaited
+// with vmcnt(0) in front of the next barrier.  Causal structure per wavefront as in the ring
+// kernel: tiles below qw0 / 64 entirely visible, tile qw0 / 64 with the block cut by the diagonal.
+// ---------------------------------------------------------------------------
+template <int D, bool BLND>
+__global__ __launch_bounds__(256, D == 128 ? 2 : 1) void flash_attn_wide_kernel(
+    const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+    const _Float16* __restrict__ V, _Float16* __restrict__ O, int heads, int L, float scale) {
+  static_assert(D == 128 || D == 256, "head sizes 128 and 256");
+  constexpr int KS = D / 16, DB = D / 32;
+  constexpr int ROWB = D * 2;             // bytes of a row
+  constexpr int CH = D / 8;               // 16-byte units of a row
+  constexpr int RPI = 1024 / ROWB;        // rows one load instruction of 1 KB covers
+  constexpr int TILE = BKEY * ROWB;       // bytes of a K (or V) tile
+  constexpr int STAGE = 2 * TILE;
+  constexpr int NDMA = D / 16;            // load instructions per wavefront and tile
+  extern __shared__ __attribute__((aligned(1024))) char smem[];  // 2 * STAGE bytes
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ql = lane & 31, g = lane >> 5;
+  const unsigned smem_base = (unsigned)(uintptr_t)smem;
+
+  const int bh = blockIdx.y;
+  const int q_blocks = (L + BQ - 1) / BQ;
+  const int qb = q_blocks - 1 - (int)blockIdx.x;  // heavy (late) query blocks first
+  const int q0 = qb * BQ;
+  const int qw0 = q0 + wave * 32, q = qw0 + ql;
+  const bool wave_active = qw0 < L;
+  int last_q = q0 + BQ - 1;
+  if (last_q > L - 1) last_q = L - 1;
+  const int nt = last_q / BKEY + 1;  // key tiles 0..nt-1 touch this query block
+
+  // ---- queries (the oldest loads in flight): lane (ql, g) holds d = 16 ks + 8 g + 0..7
+  h8 qf[KS];
+  {
+    const int qr = q < L ? q : L - 1;  // rows past the end are computed and never stored
+    const _Float16* qp = Q + ((int64_t)bh * L + qr) * D + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const h8*>(qp + ks * 16);
+  }
+
+  // ---- tile loads: wavefronts 0-1 bring the K tile, 2-3 the V tile, 32 rows each; load j of a
+  // wavefront covers rows 32 (wave % 2) + RPI j + lane / CH, lane l filling position l % CH with
+  // source unit (l % CH) ^ key(row): K key = row & 15, V key = 4 (row & 3).  RPI j contributes
+  // compile-time bits to the key, lane / CH the lane's.  Rows past the end of the sequence
+  // repeat the last row (their keys are masked, the values finite).
+  const bool brings_v = wave >= 2;
+  const char* src = (const char*)((brings_v ? V : K) + (int64_t)bh * L * D);
+  const int lrow = lane / CH;
+  const unsigned unit16 = brings_v ? (unsigned)(((lane % CH) ^ (4 * (lrow & 3))) << 4)
+                                   : (unsigned)(((lane % CH) ^ lrow) << 4);
+  auto issue_tile = [&](int t) {
+    const unsigned dst = smem_base + (unsigned)((t & 1) * STAGE) + (brings_v ? (unsigned)TILE : 0u) +
+                         (unsigned)((wave & 1) * NDMA) * 1024u;
+#pragma unroll
+    for (int j = 0; j < NDMA; ++j) {
+      int row = t * BKEY + (wave & 1) * 32 + j * RPI + lrow;
+      row = row < L ? row : L - 1;
+      const unsigned key_j = brings_v ? (unsigned)(4 * ((j * RPI) & 3)) : (unsigned)((j * RPI) & 15);
+      attn_dma16(src, (unsigned)row * (unsigned)ROWB + (unit16 ^ (key_j << 4)), dst + j * 1024);
+    }
+  };
+
+  // ---- LDS read offsets (bytes inside a tile) of this lane
+  // K fragment, k-step ks, of the 32-key block at row k: row k + ql, unit (2 ks + g) ^ (ql & 15);
+  // bits 1-3 of the unit come from ks % 8, bit 4 (head size 256) from ks / 8
+  const int tri_q = ql - 4 * g;
+  int k_off[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) k_off[ks] = ql * ROWB + (((ks * 2 + g) ^ (ql & 15)) << 4);
+  // V^T fragment of d block i, keys key0 + 4 g + 0..3: lane s = lane % 16 of its block of 16
+  // points at V[key0 + 4 g + s / 4][32 i + 16 (block % 2) + 4 (s % 4)]: unit 4 i + 2 (block % 2)
+  // + (s % 4) / 2, swizzled to 4 (i ^ (row & 3)) + ...; i % 4 varies the lane's offset, i / 4 adds
+  // 256 bytes
+  const int sl = lane & 15, vrow = 4 * g + (sl >> 2);
+  int v_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int unit = 4 * (i ^ (vrow & 3)) + 2 * ((lane >> 4) & 1) + ((sl & 3) >> 1);
+    v_off[i] = TILE + vrow * ROWB + (unit << 4) + (sl & 1) * 8;
+  }
+  const float cexp = scale * 1.4426950408889634f;
+
+  f16v oacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+  float mrun = -INFINITY, den = 0.f;
+
+  // One 64-key tile.  MODE 0: both 32-key blocks entirely visible; 1: block 0 cut by the
+  // diagonal, block 1 hidden (skipped: its weights are exactly 0); 2: block 0 visible, block 1
+  // cut by the diagonal.
+  auto step = [&](auto mode_tag, const char* buf) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr int NKB = MODE == 1 ? 1 : 2;
+    f16v s[NKB];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const h8 kf = *reinterpret_cast<const h8*>(buf + kb * 32 * ROWB + k_off[ks & 7] +
+                                                   (ks >> 3) * 256);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kb], 0, 0, 0);
+      }
+    }
+    if constexpr (MODE != 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s[NKB - 1][r] = 8 * (r >> 2) + (r & 3) <= tri_q ? s[NKB - 1][r] : -INFINITY;
+    }
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, s[kb][r]);
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+    const float mnew = bmax > mrun ? bmax : mrun;
+    const float mult = __builtin_amdgcn_exp2f((mrun - mnew) * cexp);
+    const float m2 = mnew * cexp;
+    float psum = 0.f;
+    h8 pf[NKB][2];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][8 * tt + j], cexp, -m2));
+          psum += p;
+          pf[kb][tt][j] = (_Float16)p;
+        }
+    mrun = mnew;
+    psum += __shfl_xor(psum, 32, kWave);
+    den = den * mult + psum;
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] *= mult;
+    // O^T += V^T . P^T: this lane group's keys of a 16-key step are base + 4 g + 0..3 (lo) and
+    // base + 8 + 4 g + 0..3 (hi)
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const char* vt = buf + (kb * 32 + tt * 16) * ROWB;
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+          const h4 lo = lds_read_tr16(vt + v_off[i & 3] + (i >> 2) * 256);
+          const h4 hi = lds_read_tr16(vt + v_off[i & 3] + (i >> 2) * 256 + 8 * ROWB);
+          const h8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kb][tt], oacc[i], 0, 0, 0);
+        }
+      }
+  };
+
+  const int nfull = qw0 >> 6;  // key tiles entirely below this wavefront's diagonal
+  issue_tile(0);
+  for (int t = 0; t < nt; ++t) {
+    // tile t has landed in this wavefront's part (the queries too: they are older); behind the
+    // barrier that holds for every part, and nobody reads tile t - 1 any more
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (t == 0) {
+      // the compiler cannot see the wait above; touching the query registers here makes it
+      // place its own wait for them now instead of inside the first tile
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
+    }
+    if (t + 1 < nt) issue_tile(t + 1);
+    if (wave_active && t <= nfull) {
+      const char* buf = smem + (t & 1) * STAGE;
+      if (t < nfull) step(std::integral_constant<int, 0>{}, buf);
+      else if ((qw0 & 32) == 0) step(std::integral_constant<int, 1>{}, buf);
+      else step(std::integral_constant<int, 2>{}, buf);
+    }
+  }
+
+  // ---- output, as in the streaming kernel: the two lanes of a query trade halves through the
+  // 32-lane swap and store 16 bytes each
+  const float inv = __builtin_amdgcn_rcpf(den);
+  if (q < L) {
+    int64_t row_off;
+    if (BLND) {
+      const int b = bh / heads, n = bh - b * heads;
+      row_off = (((int64_t)b * L + q) * heads + n) * D;
+    } else {
+      row_off = ((int64_t)bh * L + q) * D;
+    }
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        h4 x, y;  // d = 32 i + 16 pr + 4 g + 0..3 and the same + 8
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[j] = (_Float16)(oacc[i][8 * pr + j] * inv);
+          y[j] = (_Float16)(oacc[i][8 * pr + 4 + j] * inv);
+        }
+        const u2 xd = __builtin_bit_cast(u2, x), yd = __builtin_bit_cast(u2, y);
+        const auto r0 = __builtin_amdgcn_permlane32_swap(xd[0], yd[0], false, false);
+        const auto r1 = __builtin_amdgcn_permlane32_swap(xd[1], yd[1], false, false);
+        // g = 0: own x, then the partner's x (d + 4..7); g = 1: the partner's y, then own y
+        *reinterpret_cast<u4*>(O + row_off + i * 32 + 16 * pr + 8 * g) =
+            u4{r0[0], r1[0], r0[1], r1[1]};
+      }
+  }
+}
+
 // Deals the query chunks of a sequence of L <= 320 rows to the 8 wavefronts: chunk c costs
 // c + 1 blocks; heaviest first, each to the SIMD (wavefronts w and w + 4) with the smallest
 // load so far that still has a free slot, inside the SIMD to the lighter wavefront.
@@ -1358,6 +1585,32 @@ int launch_ring_attn(const void* q, const void* k, const void* v, void* out, int
   return 0;
 }
 
+template <int D, bool BLND>
+int launch_wide_attn(const void* q, const void* k, const void* v, void* out, int64_t BN, int heads,
+                     int L, float scale, hipStream_t st) {
+  auto kern = flash_attn_wide_kernel<D, BLND>;
+  constexpr int lds = 2 * 2 * BKEY * D * 2;  // two stages of a K tile and a V tile
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d bytes LDS): %s", lds, hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  if (BN > 65535) {  // the (batch, head) pairs go to the grid's second dimension
+    set_error("flash_attn: %lld (batch, head) pairs at head size %d: at most 65535",
+              (long long)BN, D);
+    return -2;
+  }
+  dim3 grid((unsigned)((L + BQ - 1) / BQ), (unsigned)BN);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, (const _Float16*)q, (const _Float16*)k,
+                     (const _Float16*)v, (_Float16*)out, heads, L, scale);
+  return 0;
+}
+
 template <int D, typename T>
 int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
              int heads, int L, int Lk, float scale, Dropout drop, bool blnd, hipStream_t st) {
@@ -1383,6 +1636,13 @@ int launch_d(const void* q, const void* k, const void* v, void* out, int64_t BN,
   if (const size_t lds = resident_lds_bytes(L, D)) {
     return blnd ? launch_resident<D, T, true>(q, k, v, out, BN, heads, L, scale, lds, st)
                 : launch_resident<D, T, false>(q, k, v, out, BN, heads, L, scale, lds, st);
+  }
+  if constexpr (D >= 128 && sizeof(T) == 2) {
+    // fp16, head sizes 128 and 256, longer sequences: tiles by direct loads, no staging registers
+    // (pairs in the grid's second dimension; 32-bit byte offsets inside a pair)
+    if (BN <= 65535 && (int64_t)L * D * 2 < (1ll << 31))
+      return blnd ? launch_wide_attn<D, true>(q, k, v, out, BN, heads, L, scale, st)
+                  : launch_wide_attn<D, false>(q, k, v, out, BN, heads, L, scale, st);
   }
   return blnd ? launch_tiled<D, T, true, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st)
               : launch_tiled<D, T, false, false>(q, k, v, out, BN, heads, L, Lk, scale, da, st);

@@ -588,6 +588,28 @@ def test_flash_attention_unequal_lengths(K, gpu_device, dtype, Lq, Lk):
         check_attention(host(z), want, v, dtype, f"attention Lq={Lq} Lk={Lk}")
 
 
+@pytest.mark.parametrize("D,L", [(128, 129), (128, 191), (128, 192), (128, 193), (128, 255),
+                                 (128, 256), (128, 257), (128, 300), (128, 385), (128, 700),
+                                 (256, 65), (256, 127), (256, 128), (256, 129), (256, 191),
+                                 (256, 300), (256, 513)])
+def test_flash_attention_wide_heads_fp16(K, gpu_device, D, L):
+    """fp16, head sizes 128 and 256, sequences too long for the resident variant: key tiles by
+    direct loads into two LDS stages, V read with the transposing load.  Lengths either side of
+    the 64-key tile and the 128-query block boundaries, from the shortest the kernel is picked
+    for; both output layouts; query 0 sees key 0 only."""
+    q, k, v = attn_inputs(2, 3, L, D, torch.float16, gaussian=True, seed=D + L)
+    want = O.flash_attention_v1(q, k, v)
+    args = [dev(t, gpu_device) for t in (q, k, v)]
+    print(f"wide-head attention: d={D} L={L}", flush=True)
+    z = K.flash_attention_v1(*args)
+    assert z.shape == (2, 3, L, D) and z.is_contiguous()
+    check(host(z), want, torch.float16, f"attention d={D} L={L}")
+    zm = K.flash_attention_v1(*args, merged_heads_layout=True)
+    assert zm.transpose(1, 2).is_contiguous()
+    assert torch.equal(z, zm)
+    assert np.array_equal(host(z)[:, :, 0], v[:, :, 0])
+
+
 @pytest.mark.parametrize("L", [321, 383, 384, 385, 449, 700, 1025])
 def test_flash_attention_long_sequences_fp16(K, gpu_device, L):
     """fp16, d = 64, sequences too long for the resident variant: key tiles through the ring of
