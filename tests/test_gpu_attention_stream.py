@@ -10,7 +10,9 @@ covers.  Here every call has B * N >= 64:
     kernel under Triton's CPU interpreter) placed among random pairs, so that the reference's
     vectors are compared on this kernel and not only on the few-pair ones;
   * the benchmark shape [512, 12, 300, 64]: every element of every pair against the textbook
-    attention evaluated by torch in fp32 on the GPU, the output pre-filled with NaN.
+    attention evaluated by torch in fp32 on the GPU, the output pre-filled with NaN; the same
+    check at the same bytes for head sizes 128 and 256 ([512, 6, 300, 128], [512, 3, 300, 256]),
+    which run on the wide-head kernel.
 
 Follows the reference's kernel and test: kernels.py:375-474, test.py:90-117.  Everything goes
 through ctypes -> libgptmi.so.  Tolerances: against the oracle, fp16 storage as everywhere
@@ -172,6 +174,34 @@ def test_headline_attention_every_element(K, gpu_device, layout):
     for b0 in range(0, B, 32):
         sl = slice(b0, b0 + 32)
         want, tol = attention_bound(q[sl], k[sl], v[sl], 1 / math.sqrt(D))
+        excess = (z[sl].float() - want).abs() - tol
+        n_bad += int((excess > 0).sum())
+        worst = max(worst, float(excess.max()))
+    assert n_bad == 0, f"{n_bad} elements beyond the rounding bound (worst excess {worst:.3e})"
+    assert torch.equal(z[:, :, 0], v[:, :, 0])
+
+
+@pytest.mark.parametrize("N,d", [(6, 128), (3, 256)])
+def test_wide_head_attention_every_element(K, gpu_device, N, d):
+    """The headline's bytes at head sizes 128 and 256 (the shapes `bench.py --workload ops`
+    times): every element against the textbook attention in fp32, NaN-filled output, merged-heads
+    layout (the one with the strided rows)."""
+    B, L = 512, 300
+    g = torch.Generator(device=gpu_device).manual_seed(d)
+    q, k, v = (torch.randn((B, N, L, d), generator=g, device=gpu_device).half() for _ in range(3))
+    out = torch.full((B, L, N, d), float("nan"), device=gpu_device, dtype=torch.float16)
+    lib = K._lib.load()
+    print(f"every element: attention [512, {N}, 300, {d}]", flush=True)
+    rc = lib.gptmi_flash_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, N, L, L,
+                              d, 1 / math.sqrt(d), 0.0, 1337, K._lib.GPTMI_O_BLND, K._lib.GPTMI_F16,
+                              torch.cuda.current_stream().cuda_stream)
+    K._lib.check(rc, "flash_attn")
+    z = out.transpose(1, 2)
+    assert int(torch.isnan(z).sum()) == 0, "elements never written (NaN poison left)"
+    n_bad, worst = 0, 0.0
+    for b0 in range(0, B, 32):
+        sl = slice(b0, b0 + 32)
+        want, tol = attention_bound(q[sl], k[sl], v[sl], 1 / math.sqrt(d))
         excess = (z[sl].float() - want).abs() - tol
         n_bad += int((excess > 0).sum())
         worst = max(worst, float(excess.max()))
