@@ -130,19 +130,13 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
   const int st = tid & 127;
   const bool role_k = wave < 2;
   const T* sp = role_k ? Kp : Vp;
-  int srow[NLD], scol[NLD];
-#pragma unroll
-  for (int i = 0; i < NLD; ++i) {
-    if (role_k) {
-      const int s = i * 128 + st;
-      srow[i] = s / CH;
-      scol[i] = (s % CH) * 8;
-    } else {
-      const int s = (i >> 2) * 128 + st;
-      srow[i] = (s & 15) * 4 + (i & 3);
-      scol[i] = (s >> 4) * 8;
-    }
-  }
+  // Both are a lane part plus a part that depends on i alone (128 is a multiple of CH and of 16),
+  // so two registers and compile-time increments stand for the 2 * NLD values.
+  static_assert(128 % CH == 0, "a row is at most 128 chunks");
+  const int srow0 = role_k ? st / CH : (st & 15) * 4;
+  const int scol0 = role_k ? (st % CH) * 8 : (st >> 4) * 8;
+  auto srow_of = [&](int i) { return srow0 + (role_k ? i * (128 / CH) : (i & 3)); };
+  auto scol_of = [&](int i) { return scol0 + (role_k ? 0 : (i >> 2) * 64); };
   // Two register sets: tile u travels in set u % 2.  It is requested two steps before it is
   // multiplied (during step u - 2) and written to LDS at the end of step u - 1, so a global load
   // has a whole step of arithmetic plus a barrier to arrive, not a fraction of one.  Head size
@@ -155,13 +149,13 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     const int k0 = t * BKEY;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      int row = k0 + srow[i];
+      int row = k0 + srow_of(i);
       if constexpr (UNEQ) {
-        const bool there = DG < D ? (row < Lk && scol[i] < DG) : row < Lk;
-        dst[i] = there ? Ld8<T>::load(sp + (int64_t)row * DG + scol[i]) : zero_h8();
+        const bool there = DG < D ? (row < Lk && scol_of(i) < DG) : row < Lk;
+        dst[i] = there ? Ld8<T>::load(sp + (int64_t)row * DG + scol_of(i)) : zero_h8();
       } else {
         row = row < L ? row : L - 1;
-        dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol[i]);
+        dst[i] = Ld8<T>::load(sp + (int64_t)row * D + scol_of(i));
       }
     }
   };
@@ -172,13 +166,13 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
     if (role_k) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const int key = srow[i], c = scol[i] >> 3;
+        const int key = srow_of(i), c = scol_of(i) >> 3;
         *reinterpret_cast<h8*>(ks_ + key * (D * 2) + ((c ^ (key & 7)) << 4)) = src[i];
       }
     } else {
 #pragma unroll
       for (int u = 0; u < V_UNITS; ++u) {
-        const int kg = srow[4 * u] >> 2, d0 = scol[4 * u];
+        const int kg = srow_of(4 * u) >> 2, d0 = scol_of(4 * u);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int d = d0 + j;
@@ -383,7 +377,7 @@ __global__ __launch_bounds__(256, (D == 64 && !DROP) ? 2 : 1) void flash_attn_ke
 // (L = 300: 8, 8, 7, 7 tiles).  The arithmetic per tile is that of the tiled kernel.
 // ---------------------------------------------------------------------------
 template <int D, typename T, bool BLND, int NW>
-__global__ __launch_bounds__(NW * 64, NW / 2) void flash_attn_resident_kernel(
+__global__ __launch_bounds__(NW * 64, D == 256 ? 1 : NW / 2) void flash_attn_resident_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     T* __restrict__ O, int heads, int L, float scale) {
   constexpr int CH = D / 8, KS = D / 16, DB = D / 32;
