@@ -3,12 +3,14 @@
 synthetic N(0, 0.02) weights and uniform token ids, one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload headline|batch2048|xl|ops] [--lm-head]
+                    [--workload headline|batch2048|xl|config0|ops] [--lm-head]
 
 The default (and the only line the contract asks for) is `headline`; `batch2048` is the same model
 at the max-batch memory point 2048 x 300, `xl` the GPT-2 XL shape (48 x 1600, 25 heads, batch 64 x
-seqlen 1024), `ops` times the single operators at the headline sizes (mean and median of
-event-timed repetitions, one JSON line).  `--lm-head` adds the tied LM head (logits) to the step.
+seqlen 1024), `config0` the same model at 2 x 64 tokens (bound by its launches; `--graph` times
+replays of the captured forward, `--no-ln-prologue` runs the LayerNorms as launches of their own),
+`ops` times the single operators at the headline sizes (mean and median of event-timed
+repetitions, one JSON line).  `--lm-head` adds the tied LM head (logits) to the step.
 
 A step is one forward pass (hidden state [512, 300, 768], like the reference's forward, which
 stops at the final LayerNorm) with the token ids already resident in HBM.  Prints ONE JSON
@@ -43,6 +45,9 @@ WORKLOADS = {  # name -> (architecture, batch, seqlen, description)
     "xl": (ARCH_XL, 64, 1024, "GPT-2 XL-shape forward (48 layers, d_model 1600, 25 heads x 64, FFN "
                               "6400), fp16 storage / fp32 accumulate, batch 64 x seqlen 1024"),
 }
+WORKLOADS["config0"] = (ARCH, 2, 64, "GPT-2 124M forward, fp16 storage / fp32 accumulate, batch 2 x "
+                                     "seqlen 64 (the size of the reference's CPU-runnable case: "
+                                     "bound by its launches)")
 PEAK_FP16 = 2.5e15       # MI355X dense fp16 MFMA, FLOP/s
 PEAK_HBM = 8.0e12        # bytes/s
 # HBM-side bytes of one ffn1 call come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (scaled
@@ -245,6 +250,18 @@ def bench_ops(dev):
             ops.append((f"flash attention {Bq}x{heads}x{Lq}x{d} causal",
                         (lambda a, b, c: lambda: K.flash_attention_v1(a, b, c))(qa, ka, va),
                         4 * Bq * heads * d * Lq * (Lq + 1) // 2, 4 * Bq * heads * Lq * d * 2, flush))
+    # LayerNorm followed by ffn1 + GELU as two launches and as one (the LayerNorm in the GEMM's
+    # operand prologue), at the headline's rows and at the 128 rows of a 2 x 64 batch: the one
+    # launch is for few rows, where a launch costs more than normalising a row block per column tile
+    xs = rn(128, h)
+    for rows_, xin in ((M, x), (128, xs)):
+        fl_ = 2 * rows_ * 3072 * 768
+        ops.append((f"LayerNorm -> ffn1+GELU, two launches, {rows_} rows",
+                    (lambda t: lambda: K.fused_ffn(K.fused_layer_norm(t, lw, lb), w1, bias=b1, add_gelu=True))(xin),
+                    fl_, None, None))
+        ops.append((f"LayerNorm -> ffn1+GELU, one launch (LayerNorm in the GEMM prologue), {rows_} rows",
+                    (lambda t: lambda: K.layer_norm_ffn(t, lw, lb, w1, bias=b1, add_gelu=True))(xin),
+                    fl_, None, None))
     rows = []
     for name, fn, flops, nbytes, fl in ops:
         mean, med, n = time_op(fn, fl)
@@ -281,6 +298,14 @@ def main():
                          "GEMMs are skipped (identity), which bounds what fusing them into "
                          "neighbouring kernels could return; prints an ablation line, not the "
                          "benchmark line")
+    ap.add_argument("--no-ln-prologue", action="store_true",
+                    help="small batches: run every LayerNorm as a launch of its own instead of "
+                         "inside the following GEMM (gpt.LN_PROLOGUE_MAX_ROWS = 0), for comparison")
+    ap.add_argument("--ln-prologue-under-capture", action="store_true",
+                    help="with --graph: keep the LayerNorm-in-GEMM form inside the captured graph "
+                         "(the model takes the two launches there), for comparison")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of the forward captured into a HIP graph (gpt.GraphedForward)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain copy kernel of known size (1 GiB read, 1 GiB "
                          "written) so that FETCH_SIZE / WRITE_SIZE counters of the same "
@@ -334,7 +359,14 @@ def main():
             return final_ln(x, weight, bias) if calls[0] % (2 * arch["n_layer"]) == 0 else x
 
         G.fused_layer_norm = skipped_ln
+    if args.no_ln_prologue:
+        G.LN_PROLOGUE_MAX_ROWS = 0
+    if args.ln_prologue_under_capture:
+        G.LN_PROLOGUE_UNDER_CAPTURE = True
     step = (lambda: model(ids, return_logits=True)) if args.lm_head else (lambda: model(ids))
+    if args.graph:
+        graphed = G.GraphedForward(model, ids, return_logits=args.lm_head)
+        step = lambda: graphed(ids)
 
     with torch.no_grad():
         for _ in range(args.warmup):
@@ -367,8 +399,16 @@ def main():
     tokens = batch * seqlen
     flops = forward_flops(tokens, seqlen, arch, args.lm_head)
     h = arch["n_embd"]
-    ffn1_ms = sum(a.elapsed_time(b) for a, b in ffn1_events) / max(1, len(ffn1_events))
     ffn1_flops = 2 * tokens * 4 * h * h
+    if ffn1_events:
+        ffn1_ms = sum(a.elapsed_time(b) for a, b in ffn1_events) / len(ffn1_events)
+    else:
+        # no ffn1 launch of its own was seen: the LayerNorm-prologue form (few rows) or a graph
+        # replay; time the call by itself
+        xs = torch.randn(tokens, h, device=dev).half()
+        w1 = model.blocks[0][1]._weight("ffn1_weight")
+        b1 = model.blocks[0][1].ffn1_bias.data
+        ffn1_ms = time_op(lambda: inner(xs, w1, b1, None, True, 0.0), min_ms=20.0, warm_ms=5.0)[0]
     achieved = ffn1_flops / (ffn1_ms * 1e-3) / 1e12
 
     line = {
@@ -393,7 +433,11 @@ def main():
         "mfu_note": ("executed FLOPs with the tied LM head" if args.lm_head else
                      "executed FLOPs without LM head") + " (GEMMs + causal attention) / 2.5 PFLOP/s",
         "config": {"workload": what + (", logits output (tied LM head)" if args.lm_head
-                                       else ", hidden-state output (no LM head)"),
+                                       else ", hidden-state output (no LM head)") +
+                               (", replays of a captured HIP graph" if args.graph else "") +
+                               (", LayerNorms as launches of their own" if args.no_ln_prologue else "") +
+                               (", LayerNorm-in-GEMM form kept under capture"
+                                if args.ln_prologue_under_capture else ""),
                    "tokens_per_step": tokens, "n_layer": arch["n_layer"], "n_embd": h,
                    "n_head": arch["n_head"]},
         # one ffn1 call = gemm_stream_kernel on the row tiles that fill whole rounds of the

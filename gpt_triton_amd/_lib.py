@@ -33,6 +33,11 @@ SIGNATURES = {
                                    _int, _int, _vp]),
     "gptmi_linear_qkv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                 _vp, _sz, _int, _vp]),
+    "gptmi_layernorm_linear_supported": (_int, [_i64, _i64, _int]),
+    "gptmi_layernorm_linear": (_int, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _int,
+                                      _int, _vp]),
+    "gptmi_layernorm_linear_qkv": (_int, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _i64,
+                                          _i64, _i64, _i64, _i64, _int, _vp]),
     "gptmi_flash_attn": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _f32,
                                 _u64, _int, _int, _vp]),
 }

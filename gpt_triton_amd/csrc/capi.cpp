@@ -379,6 +379,84 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q, vo
   return check_launch("linear_qkv");
 }
 
+// Shared argument checks of the two LayerNorm-prologue entry points; K = H.
+static int check_layernorm_linear(const char* what, const void* x, const void* ln_w,
+                                  const void* ln_b, const void* W, int64_t M, int64_t N,
+                                  int64_t K, int dtype) {
+  if (!x || !ln_w || !ln_b || !W || M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype)) {
+    set_error("%s: invalid argument", what);
+    return GPTMI_ERR_INVALID;
+  }
+  if (N > kMaxN) {
+    set_error("%s: N=%lld beyond %d", what, (long long)N, kMaxN);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  if (dtype != GPTMI_F16 || K > (1 << 20) || !gemm_layernorm_supported(M, (int)K)) {
+    set_error("%s: fp16 storage and a row width that is a multiple of 64 and fits the LDS panel "
+              "(gptmi_layernorm_linear_supported); use gptmi_layernorm + gptmi_linear", what);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  return GPTMI_OK;
+}
+
+int gptmi_layernorm_linear_supported(int64_t M, int64_t K, int dtype) {
+  return dtype == GPTMI_F16 && K > 0 && K <= (1 << 20) && gemm_layernorm_supported(M, (int)K) ? 1 : 0;
+}
+
+int gptmi_layernorm_linear(const void* x, const void* ln_w, const void* ln_b, float eps,
+                           const void* W_packed, const void* bias, void* out, int64_t M,
+                           int64_t N, int64_t K, int gelu, int dtype, void* stream) {
+  int rc = check_layernorm_linear("layernorm_linear", x, ln_w, ln_b, W_packed, M, N, K, dtype);
+  if (rc) return rc;
+  if (!out) {
+    set_error("layernorm_linear: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  GemmEpilogue ep = {};
+  ep.bias = bias;
+  ep.out = out;
+  ep.gelu = gelu ? 1 : 0;
+  ep.drop = Dropout{0.0f, 1337};
+  ep.qkv = false;
+  ep.f16 = true;
+  rc = launch_gemm_layernorm(x, ln_w, ln_b, eps, W_packed, M, (int)N, (int)K, ep,
+                             (hipStream_t)stream);
+  if (rc) return rc == -2 ? GPTMI_ERR_INVALID : rc;
+  return check_launch("layernorm_linear");
+}
+
+int gptmi_layernorm_linear_qkv(const void* x, const void* ln_w, const void* ln_b, float eps,
+                               const void* W_packed, const void* bias, void* q, void* k, void* v,
+                               int64_t B, int64_t L, int64_t heads, int64_t d, int64_t K,
+                               int dtype, void* stream) {
+  if (B <= 0 || L <= 0 || heads <= 0 || d <= 0 || !q || !k || !v) {
+    set_error("layernorm_linear_qkv: invalid argument");
+    return GPTMI_ERR_INVALID;
+  }
+  if (d % 8 != 0) {
+    set_error("layernorm_linear_qkv: head size %lld must be a multiple of 8", (long long)d);
+    return GPTMI_ERR_UNSUPPORTED;
+  }
+  const int64_t M = B * L, N = 3 * heads * d;
+  int rc = check_layernorm_linear("layernorm_linear_qkv", x, ln_w, ln_b, W_packed, M, N, K, dtype);
+  if (rc) return rc;
+  GemmEpilogue ep = {};
+  ep.bias = bias;
+  ep.q = q;
+  ep.k = k;
+  ep.v = v;
+  ep.L = L;
+  ep.heads = (int)heads;
+  ep.d = (int)d;
+  ep.drop = Dropout{0.0f, 1337};
+  ep.qkv = true;
+  ep.f16 = true;
+  rc = launch_gemm_layernorm(x, ln_w, ln_b, eps, W_packed, M, (int)N, (int)K, ep,
+                             (hipStream_t)stream);
+  if (rc) return rc == -2 ? GPTMI_ERR_INVALID : rc;
+  return check_launch("layernorm_linear_qkv");
+}
+
 int gptmi_flash_attn(const void* q, const void* k, const void* v, void* out, int64_t B,
                      int64_t N, int64_t Lq, int64_t Lk, int64_t d, float scale, float p,
                      uint64_t seed, int olayout, int dtype, void* stream) {

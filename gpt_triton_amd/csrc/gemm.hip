@@ -44,8 +44,11 @@
 // end) picks kernel and configuration.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
+#include "layernorm.h"
 
 namespace gptmi {
 
@@ -66,6 +69,16 @@ struct EpiDev {
   int vec8_ok; // fp16 output: N, head size and the output pointers also allow 16-byte stores
   int m_off;   // head-major scatter: row 0 of this launch is row m_off of the [B*L] token rows
   DropoutArgs drop;  // p > 0: dropout between GELU and residual (predicated epilogue only)
+};
+
+// LayerNorm in the operand prologue (gemm_kernel<..., LNA = true>): weight, bias, epsilon and
+// the lanes per row the LayerNorm kernel would use for rows of this width (the sums are then
+// formed in the same order and the normalised operand has the same bits as that kernel's output).
+struct LnArgs {
+  const void* w;
+  const void* b;
+  float eps;
+  int lpr;
 };
 
 // Direct global->LDS load of 16 bytes per lane: lane l's bytes land at LDS
@@ -645,13 +658,19 @@ __device__ __forceinline__ int xcd_tile(int pid, int num_tiles) {
 
 // WPE = wavefronts per SIMD the register allocation must leave room for (two
 // 4-wavefront workgroups per CU need 2).
+// LNA: the A operand is LayerNorm(x).  The workgroup normalises its BM rows of x [M][Kp] once
+// (fp32 statistics, the arithmetic and summation order of layernorm_vec_kernel, rounded to fp16)
+// into an LDS panel that holds all k-tiles of those rows, and only the weights travel through
+// the stages.  For few rows (the launcher's choice): the normalised matrix never goes to memory
+// and its kernel launch is gone; every column tile of a row block normalises the rows again.
 template <int BM, int BN, int WM, int WN, int BKS, int NST, int WPE, typename T, bool QKV,
-          bool RESLDS = false>
+          bool RESLDS = false, bool LNA = false>
 __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     const _Float16* __restrict__ A, const _Float16* __restrict__ Bt, int M, int N, int Kp,
-    int tiles_m, int tiles_n, int group_w, EpiDev ep) {
+    int tiles_m, int tiles_n, int group_w, EpiDev ep, LnArgs ln) {
   static_assert(BKS == 32 || BKS == 64, "k-step of 32 or 64");
   static_assert(NST >= 2, "at least double buffering");
+  static_assert(!LNA || (BKS == 64 && !RESLDS && sizeof(T) == 2), "LayerNorm prologue: fp16, k-step 64");
   constexpr int T_ = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int MB = TM / 32, NB = TN / 32;
@@ -659,9 +678,12 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   constexpr int CPR = ROWB / 16;           // 16-byte chunks per row (4 or 8)
   constexpr int CSH = CPR == 8 ? 3 : 2;    // log2(CPR)
   constexpr int KSH = CPR == 8 ? 1 : 2;    // swizzle key = (row >> KSH) & (CPR-1)
-  constexpr int A_IT = BM * CPR / T_, B_IT = BN * CPR / T_;
+  // LNA: no A loads, the stages hold weight rows only, the panel lies behind the stages
+  constexpr int A_IT = LNA ? 0 : BM * CPR / T_, B_IT = BN * CPR / T_;
+  constexpr int A_N = A_IT ? A_IT : 1;     // array extent
   constexpr int LPT = A_IT + B_IT;         // direct loads per thread per k-tile
-  constexpr int STAGE = (BM + BN) * ROWB;
+  constexpr int B_AT = LNA ? 0 : BM * ROWB;  // byte offset of the weight rows inside a stage
+  constexpr int STAGE = B_AT + BN * ROWB;
   constexpr int KS = BKS / 16;             // MFMA k-steps per tile
   static_assert(BM * CPR % T_ == 0 && BN * CPR % T_ == 0, "tile/threads mismatch");
   static_assert(TM % 32 == 0 && TN % 64 == 0, "wave tile must be 32 x 64 aligned");
@@ -695,7 +717,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   // 16-byte slot s of an operand tile: row s / CPR, position s % CPR, which
   // holds source chunk (s % CPR) ^ key(row).  Rows past the matrix edge re-read
   // the last row (their products are never stored).
-  const char* a_src[A_IT];
+  const char* a_src[A_N];
   const char* b_src[B_IT];
 #pragma unroll
   for (int it = 0; it < A_IT; ++it) {
@@ -715,7 +737,7 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
       __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + (unsigned)wave * 1024u);
   auto issue = [&](int kt) {
     const unsigned as = wave_off + (kt % NST) * STAGE;
-    const unsigned bs = as + BM * ROWB;
+    const unsigned bs = as + B_AT;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it)
       lds_dma16(a_src[it] + (size_t)kt * ROWB, as + it * T_ * 16);
@@ -727,8 +749,8 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   // one of the A_IT + B_IT loads of k-tile kt (the A loads come first)
   auto issue_one = [&](int kt, int n) {
     const unsigned as = wave_off + (kt % NST) * STAGE;
-    if (n < A_IT) lds_dma16(a_src[n] + (size_t)kt * ROWB, as + n * T_ * 16);
-    else lds_dma16(b_src[n - A_IT] + (size_t)kt * ROWB, as + BM * ROWB + (n - A_IT) * T_ * 16);
+    if (n < A_IT) lds_dma16(a_src[n < A_IT ? n : 0] + (size_t)kt * ROWB, as + n * T_ * 16);
+    else lds_dma16(b_src[n - A_IT] + (size_t)kt * ROWB, as + B_AT + (n - A_IT) * T_ * 16);
   };
 
   f16v acc[NB][MB];
@@ -742,14 +764,17 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
   // fragment read offsets (bytes) inside a stage
   const int frow = lane & 31, fhalf = lane >> 5, fkey = (frow >> KSH) & (CPR - 1);
   const int a_row_off = (wm * TM + frow) * ROWB;
-  const int b_row_off = BM * ROWB + (wn * TN + frow) * ROWB;
+  const int b_row_off = B_AT + (wn * TN + frow) * ROWB;
+  // LNA: k-tile kt of the normalised rows, laid out like the A part of a stage
+  const char* panel = smem + NST * STAGE;
   h8 af[2][MB], bf[2][NB];
   auto read_frags = [&](int kt, int ks, int slot) {
     const char* st = smem + (kt % NST) * STAGE;
+    const char* sa = LNA ? panel + kt * (BM * ROWB) : st;
     const int choff = ((ks * 2 + fhalf) ^ fkey) << 4;
 #pragma unroll
     for (int j = 0; j < MB; ++j)
-      af[slot][j] = *reinterpret_cast<const h8*>(st + a_row_off + j * 32 * ROWB + choff);
+      af[slot][j] = *reinterpret_cast<const h8*>(sa + a_row_off + j * 32 * ROWB + choff);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
       bf[slot][i] = *reinterpret_cast<const h8*>(st + b_row_off + i * 32 * ROWB + choff);
@@ -814,10 +839,111 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
 #pragma unroll
   for (int s = 0; s < NST; ++s)
     if (s < KT) issue(s);
-  // tile 0 must have landed; up to NST-1 younger tiles stay in flight
-  if (KT >= NST) wait_vmcnt<(NST - 1) * LPT>();
-  else wait_vmcnt<0>();
-  asm volatile("s_barrier" ::: "memory");
+  if constexpr (LNA) {
+    // The rows of this tile, normalised, into the panel: chunk c of row r goes to k-tile c / 8,
+    // position (c % 8) ^ key(r) of the row's 128 bytes.  A row is spread over LPR lanes as in
+    // layernorm_vec_kernel (T_ / LPR rows per pass); rows past the end repeat the last row.
+    const int H = Kp, nchunks = H >> 3;
+    auto ln_rows = [&](auto lpr_tag, auto ch_tag) {
+      constexpr int LPR = decltype(lpr_tag)::value, CH = decltype(ch_tag)::value;
+      constexpr int RPP = T_ / LPR;
+      const int ll = tid & (LPR - 1), rsub = tid / LPR;
+      const h8* wv = reinterpret_cast<const h8*>(ln.w);
+      const h8* bv = reinterpret_cast<const h8*>(ln.b);
+      // the parameters of the lane's chunks: held across the rows, unless the rows are so long
+      // that they and a row do not fit the registers together (then fetched per row, from L1)
+      constexpr bool HOLD = CH <= 4;
+      h8 tw[CH], tb[CH];
+      if constexpr (HOLD) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+          const int c = ll + i * LPR;
+          if (c < nchunks) {
+            tw[i] = wv[c];
+            tb[i] = bv[c];
+          }
+        }
+      }
+      // G rows per thread group are requested together, so that a workgroup waits for memory
+      // BM / (RPP * G) times and not once per row (G * CH 16-byte registers hold them)
+      constexpr int PASSES = BM / RPP;
+      constexpr int G0 = CH <= 3 ? 8 : CH <= 4 ? 4 : 2, G = G0 < PASSES ? G0 : PASSES;
+      static_assert(PASSES % G == 0, "row groups");
+      for (int p0 = 0; p0 < PASSES; p0 += G) {
+        h8 t[G][CH];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          int row = m0 + (p0 + g) * RPP + rsub;
+          row = row < M ? row : M - 1;
+          const h8* xr = reinterpret_cast<const h8*>(A + (size_t)row * Kp);
+#pragma unroll
+          for (int i = 0; i < CH; ++i) {
+            const int c = ll + i * LPR;
+            if (c < nchunks) t[g][i] = xr[c];
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int r = (p0 + g) * RPP + rsub;
+          float v[CH][8];
+          float sum = 0.f;
+#pragma unroll
+          for (int i = 0; i < CH; ++i) {
+            const int c = ll + i * LPR;
+            if (c < nchunks) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                v[i][j] = (float)t[g][i][j];
+                sum += v[i][j];
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+            }
+          }
+          float mean, rstd;
+          layernorm_stats<CH, 8, LPR>(v, sum, ll, nchunks, H, ln.eps, mean, rstd);
+#pragma unroll
+          for (int i = 0; i < CH; ++i) {
+            const int c = ll + i * LPR;
+            if (c < nchunks) {
+              if constexpr (!HOLD) {
+                tw[i] = wv[c];
+                tb[i] = bv[c];
+              }
+              h8 to;
+#pragma unroll
+              for (int j = 0; j < 8; ++j)
+                to[j] = (_Float16)layernorm_apply(v[i][j], mean, rstd, (float)tw[i][j],
+                                                  (float)tb[i][j]);
+              *reinterpret_cast<h8*>(const_cast<char*>(panel) + (c >> 3) * (BM * ROWB) + r * ROWB +
+                                     (((c & 7) ^ ((r >> KSH) & 7)) << 4)) = to;
+            }
+          }
+        }
+      }
+    };
+    const int need = (nchunks + ln.lpr - 1) / ln.lpr;  // chunks per lane; the launcher checked <= 8
+#define GPTMI_LN_ROWS(L)                                                            \
+  do {                                                                              \
+    using LT = std::integral_constant<int, L>;                                      \
+    if (need <= 1) ln_rows(LT{}, std::integral_constant<int, 1>{});                 \
+    else if (need <= 2) ln_rows(LT{}, std::integral_constant<int, 2>{});            \
+    else if (need <= 3) ln_rows(LT{}, std::integral_constant<int, 3>{});            \
+    else if (need <= 4) ln_rows(LT{}, std::integral_constant<int, 4>{});            \
+    else ln_rows(LT{}, std::integral_constant<int, 8>{});                           \
+  } while (0)
+    if (ln.lpr == 32) GPTMI_LN_ROWS(32);
+    else GPTMI_LN_ROWS(64);
+#undef GPTMI_LN_ROWS
+    // panel written, the first weight k-tiles landed (the compiler's barrier waits for both)
+    __syncthreads();
+  } else {
+    // tile 0 must have landed; up to NST-1 younger tiles stay in flight
+    if (KT >= NST) wait_vmcnt<(NST - 1) * LPT>();
+    else wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+  }
   read_frags(0, 0, 0);
 
   for (int kt = 0; kt < KT; ++kt) {
@@ -920,7 +1046,34 @@ int launch_cfg(const void* A, const void* Bt, int64_t M, int N, int Kp, const Ep
   const int group_w = column_group(tiles_n, BN, Kp);
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(WM * WN * 64), smem, st,
                      (const _Float16*)A, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n,
-                     group_w, ep);
+                     group_w, ep, LnArgs{});
+  return 0;
+}
+
+// The LayerNorm-prologue form: 32 x 128 tiles, 2 wavefronts, three stages of weight rows
+// (48 KB) and the panel of the tile's 32 normalised rows (64 * Kp bytes) behind them.
+constexpr int LNA_BM = 32, LNA_BN = 128, LNA_NST = 3;
+inline size_t lna_lds_bytes(int Kp) { return (size_t)LNA_NST * LNA_BN * 128 + (size_t)LNA_BM * Kp * 2; }
+
+template <bool QKV>
+int launch_lna(const void* x, const void* Bt, int64_t M, int N, int Kp, const EpiDev& ep,
+               const LnArgs& ln, hipStream_t st) {
+  auto kern = gemm_kernel<LNA_BM, LNA_BN, 1, 2, 64, LNA_NST, 2, _Float16, QKV, false, true>;
+  static bool attr_done = false;  // idempotent; a race only repeats the call
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(160 KB LDS): %s", hipGetErrorString(e));
+      return -4;
+    }
+    attr_done = true;
+  }
+  const int tiles_m = (int)((M + LNA_BM - 1) / LNA_BM), tiles_n = (N + LNA_BN - 1) / LNA_BN;
+  const int group_w = column_group(tiles_n, LNA_BN, Kp);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(128), lna_lds_bytes(Kp), st,
+                     (const _Float16*)x, (const _Float16*)Bt, (int)M, N, Kp, tiles_m, tiles_n,
+                     group_w, ep, ln);
   return 0;
 }
 
@@ -1754,8 +1907,8 @@ int launch_shape(const void* A, const void* Bt, int64_t M, int N, int Kp, const 
 
 }  // namespace
 
-int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const GemmEpilogue& e,
-                hipStream_t st) {
+// The device-side epilogue description of a launch, or a negative error code.
+static int make_epi(const GemmEpilogue& e, int64_t M, int N, EpiDev& ep) {
   if (M >= (1ll << 31) - 512) {
     set_error("gemm: M=%lld does not fit the kernel's 32-bit row index", (long long)M);
     return -2;
@@ -1764,7 +1917,7 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const G
     set_error("gemm qkv epilogue: head size %d must be a multiple of 4", e.d);
     return -2;
   }
-  EpiDev ep = {};
+  ep = EpiDev{};
   ep.bias = e.bias;
   ep.residual = e.residual;
   ep.out = e.out;
@@ -1785,11 +1938,43 @@ int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const G
   auto aligned16 = [&](const void* p) { return ((uintptr_t)p & 15) == 0; };
   ep.vec8_ok = vec && e.f16 && (N % 8) == 0 && aligned16(e.out) && aligned16(e.q) &&
                aligned16(e.k) && aligned16(e.v) && (!e.qkv || (e.d % 8) == 0);
+  return 0;
+}
+
+int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp, const GemmEpilogue& e,
+                hipStream_t st) {
+  EpiDev ep;
+  if (const int rc = make_epi(e, M, N, ep)) return rc;
   if (e.f16)
     return e.qkv ? launch_shape<_Float16, true>(A, Bt, M, N, Kp, ep, st)
                  : launch_shape<_Float16, false>(A, Bt, M, N, Kp, ep, st);
   return e.qkv ? launch_shape<float, true>(A, Bt, M, N, Kp, ep, st)
                : launch_shape<float, false>(A, Bt, M, N, Kp, ep, st);
+}
+
+bool gemm_layernorm_supported(int64_t M, int H) {
+  if (H <= 0 || H % 64 != 0 || M <= 0) return false;
+  const int nchunks = H / 8, lpr = lanes_per_row(nchunks);
+  return (nchunks + lpr - 1) / lpr <= 8 && lna_lds_bytes(H) <= 160 * 1024;
+}
+
+int launch_gemm_layernorm(const void* x, const void* ln_w, const void* ln_b, float eps,
+                          const void* Bt, int64_t M, int N, int H, const GemmEpilogue& e,
+                          hipStream_t st) {
+  if (!e.f16 || e.residual != nullptr || e.drop.p > 0.f || !gemm_layernorm_supported(M, H)) {
+    set_error("gemm with LayerNorm prologue: fp16, no residual, no dropout, H=%d a multiple of "
+              "64 whose 32-row panel fits the LDS", H);
+    return -2;
+  }
+  if ((((uintptr_t)x | (uintptr_t)ln_w | (uintptr_t)ln_b | (uintptr_t)Bt) & 15) != 0) {
+    set_error("gemm with LayerNorm prologue: x, the LayerNorm parameters and W must be 16-byte aligned");
+    return -2;
+  }
+  EpiDev ep;
+  if (const int rc = make_epi(e, M, N, ep)) return rc;
+  const LnArgs ln = {ln_w, ln_b, eps, lanes_per_row(H / 8)};
+  return e.qkv ? launch_lna<true>(x, Bt, M, N, H, ep, ln, st)
+               : launch_lna<false>(x, Bt, M, N, H, ep, ln, st);
 }
 
 }  // namespace gptmi

@@ -49,6 +49,16 @@ struct GemmEpilogue {
 int launch_gemm(const void* A, const void* Bt, int64_t M, int N, int Kp,
                 const GemmEpilogue& ep, hipStream_t st);
 
+// The same product with A = LayerNorm(x; ln_w, ln_b, eps), x [M][H] fp16 with H = K a multiple
+// of 64: every workgroup normalises the rows of its tile in its operand prologue (the bits of
+// launch_layernorm's output) and the normalised matrix never goes to memory.  fp16, no residual,
+// no dropout; meant for few rows, where a LayerNorm launch costs more than normalising the rows
+// once per column tile.  gemm_layernorm_supported says whether (M, H) is taken.
+bool gemm_layernorm_supported(int64_t M, int H);
+int launch_gemm_layernorm(const void* x, const void* ln_w, const void* ln_b, float eps,
+                          const void* Bt, int64_t M, int N, int H, const GemmEpilogue& ep,
+                          hipStream_t st);
+
 // q, out: L rows per (batch, head); k, v: Lk rows.
 int launch_flash_attn(const void* q, const void* k, const void* v, void* out,
                       int64_t B, int64_t N, int64_t L, int64_t Lk, int d, float scale,

@@ -2,6 +2,7 @@
 // operand packers of the GEMM.  One wavefront owns one row; a row is held in
 // registers between its passes so HBM sees one read and one write per element.
 #include "common.h"
+#include "layernorm.h"
 #include "launch.h"
 
 namespace gptmi {
@@ -84,41 +85,6 @@ __global__ __launch_bounds__(256) void embed_dropout_kernel(
   }
 }
 
-// The arithmetic of one LayerNorm row, shared by layernorm_vec_kernel and embed_layernorm_kernel
-// so that the two give the same bits: fp32 mean, then the centred biased variance, then
-// (x - mean) * rstd * w + b.  Contraction is spelled out (fmaf where a multiply-add is fused,
-// none elsewhere): left to the compiler, the two kernels were fused differently.
-#pragma clang fp contract(off)
-template <int CH, int VN, int LPR>
-__device__ __forceinline__ void layernorm_stats(const float (&v)[CH][VN], float s, int lane,
-                                                int nchunks, int H, float eps, float& mean,
-                                                float& rstd) {
-  mean = group_sum<LPR>(s) / (float)H;
-  float q = 0.f;
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    if (lane + i * LPR < nchunks) {
-#pragma unroll
-      for (int j = 0; j < VN; ++j) {
-        const float d = v[i][j] - mean;
-        q = __builtin_fmaf(d, d, q);
-      }
-    }
-  }
-  const float var = group_sum<LPR>(q) / (float)H;
-  rstd = 1.0f / sqrtf(var + eps);
-}
-__device__ __forceinline__ float layernorm_apply(float x, float mean, float rstd, float w, float b) {
-  const float z = (x - mean) * rstd;
-  float r = __builtin_fmaf(z, w, b);
-  // The result is an fp32 number that the caller rounds to the storage type (the reference's
-  // fp32 arithmetic followed by a cast).  Without this fence the compiler may merge the
-  // multiply-add and the conversion into one mixed-precision instruction that rounds the exact
-  // result once, straight to fp16 -- in some kernels and not in others.
-  asm("" : "+v"(r));
-  return r;
-}
-#pragma clang fp contract(fast)
 
 // ---------------------------------------------------------------------------
 // LayerNorm (reference: fused_layer_norm_kernel, kernels.py:104-145): fp32
@@ -390,13 +356,6 @@ __global__ __launch_bounds__(256) void pack_transpose_kernel(const T* __restrict
 // ---------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------
-// Lanes per row for rows of `nchunks` 16-byte chunks: 32 if that leaves fewer idle lane slots
-// than 64 (96 chunks: 3 passes of 32 against 2 passes of 64 with a quarter empty).
-static inline int lanes_per_row(int nchunks) {
-  const int slots32 = (nchunks + 31) / 32 * 32, slots64 = (nchunks + 63) / 64 * 64;
-  return slots32 < slots64 ? 32 : 64;
-}
-
 template <typename T>
 static int launch_embed_t(const int64_t* ids, const void* wte, const void* wpe,
                           void* out, int64_t rows, int64_t L, int64_t V, int H, Dropout drop,

@@ -22,7 +22,23 @@ import torch
 import torch.nn as nn
 
 from .kernels import (flash_attention_v1, fused_embeddings, fused_embeddings_layer_norm, fused_ffn,
-                      fused_layer_norm, lm_head, matmul_and_split_qkv, pack_lm_head, pack_weight)
+                      fused_layer_norm, layer_norm_ffn, layer_norm_linear_supported,
+                      layer_norm_matmul_and_split_qkv, lm_head, matmul_and_split_qkv, pack_lm_head,
+                      pack_weight)
+
+# Up to this many token rows the blocks run their LayerNorm inside the following GEMM
+# (layer_norm_ffn, layer_norm_matmul_and_split_qkv: one launch instead of two, same bits): such
+# a forward is bound by its launches.  Above, the LayerNorm kernel and the big-tile GEMMs are
+# faster -- the fused form normalises a row block once per column tile and runs on small tiles --
+# and so are the two launches inside a captured graph, where a launch costs next to nothing.
+LN_PROLOGUE_MAX_ROWS = 1024
+LN_PROLOGUE_UNDER_CAPTURE = False  # measurement switch (bench.py --ln-prologue-under-capture)
+
+
+def _ln_in_gemm(x, weight):
+    return (x.numel() // x.shape[-1] <= LN_PROLOGUE_MAX_ROWS and
+            layer_norm_linear_supported(x, weight) and
+            (LN_PROLOGUE_UNDER_CAPTURE or not torch.cuda.is_current_stream_capturing()))
 
 # dense fp16/bf16 tensor throughput, FLOP/s
 GPU_TO_FLOPS = {
@@ -96,10 +112,15 @@ class FusedAttention(nn.Module):
         p = self.dropout_prob if self.training else 0.0
         skip = x
         y = normed
-        if y is None:
-            y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
-        q, k, v = matmul_and_split_qkv(y, self._weight("c_attn_weight"), self.c_attn_bias.data,
-                                       self.num_heads)
+        w_attn = self._weight("c_attn_weight")
+        if y is None and p == 0.0 and _ln_in_gemm(x, w_attn):
+            q, k, v = layer_norm_matmul_and_split_qkv(x, self.layer_norm_weight.data,
+                                                      self.layer_norm_bias.data, w_attn,
+                                                      self.c_attn_bias.data, self.num_heads)
+        else:
+            if y is None:
+                y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+            q, k, v = matmul_and_split_qkv(y, w_attn, self.c_attn_bias.data, self.num_heads)
         # [B, N, L, d] values in a [B, L, N, d] buffer: the head merge below copies nothing
         y = flash_attention_v1(q, k, v, dropout_prob=p, merged_heads_layout=True)
         y = y.transpose(1, 2).contiguous().view(skip.shape)
@@ -140,9 +161,14 @@ class FusedMLP(nn.Module):
     def forward(self, x):
         p = self.dropout_prob if self.training else 0.0
         skip = x
-        y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
-        y = fused_ffn(y, self._weight("ffn1_weight"), bias=self.ffn1_bias.data, residual=None,
-                      add_gelu=True, dropout_prob=p)
+        w1 = self._weight("ffn1_weight")
+        if p == 0.0 and _ln_in_gemm(x, w1):
+            y = layer_norm_ffn(x, self.layer_norm_weight.data, self.layer_norm_bias.data, w1,
+                               bias=self.ffn1_bias.data, add_gelu=True)
+        else:
+            y = fused_layer_norm(x, self.layer_norm_weight.data, self.layer_norm_bias.data)
+            y = fused_ffn(y, w1, bias=self.ffn1_bias.data, residual=None, add_gelu=True,
+                          dropout_prob=p)
         return fused_ffn(y, self._weight("ffn2_weight"), bias=self.ffn2_bias.data, residual=skip,
                          add_gelu=False, dropout_prob=p)
 

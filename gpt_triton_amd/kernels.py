@@ -343,6 +343,74 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
     return q, k, v
 
 
+def layer_norm_linear_supported(x, weight):
+    """True where `layer_norm_ffn` / `layer_norm_matmul_and_split_qkv` take these operands: fp16,
+    a packed weight image, a row width the kernel's LDS panel holds."""
+    if not isinstance(weight, PackedWeight) or x.dtype != torch.float16:
+        return False
+    H = x.shape[-1]
+    return bool(_lib.load().gptmi_layernorm_linear_supported(x.numel() // H, H, _lib.GPTMI_F16))
+
+
+def _check_layer_norm_linear(x, ln_weight, ln_bias, weight, bias, what):
+    assert x.is_contiguous() and ln_weight.is_contiguous() and ln_bias.is_contiguous()
+    assert ln_weight.shape == ln_bias.shape == (x.shape[-1],)
+    assert x.shape[-1] == weight.shape[0]
+    if not isinstance(weight, PackedWeight):
+        raise NotImplementedError(f"{what}: takes the packed image of the weight (pack_weight)")
+    if not (x.dtype == ln_weight.dtype == ln_bias.dtype == weight.dtype == torch.float16):
+        raise NotImplementedError(f"{what}: fp16 operands only")
+    if bias is not None:
+        assert bias.is_contiguous() and bias.shape == (weight.shape[1],)
+        if bias.dtype != x.dtype:
+            raise TypeError(f"{what}: bias is {bias.dtype} but x is {x.dtype}")
+    return _on_gpu(x, ln_weight, ln_bias, weight, bias)
+
+
+@torch.no_grad()
+def layer_norm_ffn(x, ln_weight, ln_bias, weight, bias=None, add_gelu=False):
+    """gelu?(fused_layer_norm(x, ln_weight, ln_bias) @ weight + bias) in one launch: the
+    LayerNorm runs in the GEMM's operand prologue (the fusion marked as to do in the reference,
+    kernels.py:132-133) and gives the bits of fused_layer_norm followed by fused_ffn.  Meant for
+    few rows; `weight` is a `pack_weight` image, fp16 only (NotImplementedError otherwise, and
+    for row widths `layer_norm_linear_supported` turns down)."""
+    dev = _check_layer_norm_linear(x, ln_weight, ln_bias, weight, bias, "layer_norm_ffn")
+    K, N = weight.shape
+    M = x.numel() // K
+    z = torch.empty((*x.shape[:-1], N), device=dev, dtype=x.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_layernorm_linear(x.data_ptr(), ln_weight.data_ptr(), ln_bias.data_ptr(),
+                                        1e-5, weight.data_ptr(), _ptr(bias), z.data_ptr(), M, N, K,
+                                        int(bool(add_gelu)), _lib.GPTMI_F16, _stream())
+    _lib.check(rc, "layer_norm_ffn")
+    return z
+
+
+@torch.no_grad()
+def layer_norm_matmul_and_split_qkv(x, ln_weight, ln_bias, weight, bias, num_heads):
+    """matmul_and_split_qkv(fused_layer_norm(x, ln_weight, ln_bias), weight, bias, num_heads) in
+    one launch, same bits; see `layer_norm_ffn`.  x [B, L, h]; head size a multiple of 8."""
+    dev = _check_layer_norm_linear(x, ln_weight, ln_bias, weight, bias,
+                                   "layer_norm_matmul_and_split_qkv")
+    batch_size, seqlen, K = x.shape
+    hidden_size = weight.shape[1] // 3
+    assert weight.shape[1] == 3 * hidden_size and hidden_size % num_heads == 0
+    head_size = hidden_size // num_heads
+    shape = (batch_size, num_heads, seqlen, head_size)
+    q = torch.empty(shape, device=dev, dtype=x.dtype)
+    k = torch.empty(shape, device=dev, dtype=x.dtype)
+    v = torch.empty(shape, device=dev, dtype=x.dtype)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.gptmi_layernorm_linear_qkv(x.data_ptr(), ln_weight.data_ptr(), ln_bias.data_ptr(),
+                                            1e-5, weight.data_ptr(), _ptr(bias), q.data_ptr(),
+                                            k.data_ptr(), v.data_ptr(), batch_size, seqlen,
+                                            num_heads, head_size, K, _lib.GPTMI_F16, _stream())
+    _lib.check(rc, "layer_norm_matmul_and_split_qkv")
+    return q, k, v
+
+
 @torch.no_grad()
 def flash_attention_v1(q, k, v, dropout_prob=0.0, *, merged_heads_layout=False):
     """Causal softmax(q k^T / sqrt(d)) v for q, k, v [B, N, L, d] -> [B, N, L, d].

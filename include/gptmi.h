@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define GPTMI_VERSION 101 /* major*10000 + minor*100 + patch */
+#define GPTMI_VERSION 102 /* major*10000 + minor*100 + patch */
 
 /* Size of the scratch array built into the library for gptmi_linear_static (8 MiB). */
 #define GPTMI_STATIC_SCRATCH_BYTES (8u << 20)
@@ -222,6 +222,33 @@ int gptmi_linear_qkv(const void* x, const void* W, const void* bias, void* q,
                      void* k, void* v, int64_t B, int64_t L, int64_t heads,
                      int64_t d, int64_t K, int wlayout, void* workspace,
                      size_t workspace_bytes, int dtype, void* stream);
+
+/*
+ * out = gelu?(LayerNorm(x; ln_w, ln_b, eps) @ W + bias), and the same with the head-major
+ * scatter of gptmi_linear_qkv: the LayerNorm runs in the GEMM's operand prologue.  Every
+ * workgroup normalises the 32 rows of its tile (fp32 statistics, the arithmetic of
+ * gptmi_layernorm: the operand has the bits of that call's output) into LDS; the normalised
+ * matrix never goes to memory and its kernel launch is gone.  Each column tile of a row block
+ * normalises the rows again, so this pays for FEW rows, where a forward is bound by its launches
+ * (the callers in gpt.py use it below a row count and gptmi_layernorm + gptmi_linear above).
+ *
+ * Replaces the pairs fused_layer_norm -> matmul_and_split_qkv (gpt.py:40-41) and
+ * fused_layer_norm -> fused_ffn (gpt.py:92-93) of the reference's blocks: the fusion its
+ * author marks as to do at kernels.py:132-133.
+ *   x [M][K] fp16 (M = B*L)   ln_w, ln_b [K]   W_packed: the image gptmi_pack_weight writes
+ *   bias [N] or NULL          K a multiple of 64; fp16 storage only; no residual, no dropout
+ * gptmi_layernorm_linear_supported(M, K, dtype) = 1 where the calls take these sizes; they
+ * return GPTMI_ERR_UNSUPPORTED elsewhere (K not a multiple of 64 or beyond what the 32-row
+ * panel of 64*K bytes leaves of the LDS beside 48 KB of weight stages; fp32 storage).
+ */
+int gptmi_layernorm_linear_supported(int64_t M, int64_t K, int dtype);
+int gptmi_layernorm_linear(const void* x, const void* ln_w, const void* ln_b, float eps,
+                           const void* W_packed, const void* bias, void* out, int64_t M,
+                           int64_t N, int64_t K, int gelu, int dtype, void* stream);
+int gptmi_layernorm_linear_qkv(const void* x, const void* ln_w, const void* ln_b, float eps,
+                               const void* W_packed, const void* bias, void* q, void* k,
+                               void* v, int64_t B, int64_t L, int64_t heads, int64_t d,
+                               int64_t K, int dtype, void* stream);
 
 /*
  * out = softmax(causal(q k^T * scale)) v, mask "key index <= query index".

@@ -37,7 +37,7 @@ def test_header_symbols_are_exported_and_bound(lib):
 
 
 def test_version_and_error_string(lib):
-    assert lib.gptmi_version() == 101
+    assert lib.gptmi_version() == 102
     assert isinstance(lib.gptmi_last_error(), bytes)
 
 
