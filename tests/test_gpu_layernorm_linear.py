@@ -58,7 +58,7 @@ def operands(M, H, N, seed):
 
 
 @pytest.mark.parametrize("M,H,N,gelu,bias", [
-    (128, 768, 3072, True, True),    # GPT-2's ffn1 at BASELINE's configuration 0 (2 x 64 tokens)
+    (128, 768, 3072, True, True),    # GPT-2's ffn1 at benchmark configuration 0 (2 x 64 tokens)
     (128, 768, 768, False, True),
     (1, 768, 2304, False, True),     # one row: 31 rows of the tile repeat it
     (33, 768, 100, True, False),     # a second row tile with one row, a column tile cut at 100
@@ -144,7 +144,7 @@ def test_layer_norm_linear_turns_down_what_it_does_not_hold(K, gpu_device):
 
 
 def test_model_same_bits_with_and_without_the_prologue(gpu_device, monkeypatch):
-    """FusedGPT at BASELINE's configuration 0 (2 x 64 tokens, the 124M architecture, fp16):
+    """FusedGPT at benchmark configuration 0 (2 x 64 tokens, the 124M architecture, fp16):
     hidden state and logits with the LayerNorms inside the GEMMs and with them as launches of
     their own are the same bits, and both stay within the model tolerance of the oracle."""
     from gpt_triton_amd import gpt as G
