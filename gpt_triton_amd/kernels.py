@@ -49,7 +49,28 @@ def _on_gpu(*tensors):
 
 
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    # torch's current stream on the current device as the raw hipStream_t; the direct binding
+    # costs a fraction of building a torch.cuda.Stream object per operator call
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _device(dev):
+    """Context in which `dev` is the current device: nothing to do (and nothing to pay per call)
+    when it already is, torch's guard otherwise."""
+    if dev.index is None or dev.index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(dev)
 
 
 def _ptr(t):
@@ -88,7 +109,7 @@ def pack_weight(weight):
     K_, N = weight.shape
     lib = _lib.load()
     buf = torch.empty(lib.gptmi_packed_weight_bytes(N, K_), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_pack_weight(weight.data_ptr(), buf.data_ptr(), N, K_, _lib.GPTMI_W_KN,
                                    _dtype_code(weight, "pack_weight"), _stream())
     _lib.check(rc, "pack_weight")
@@ -108,7 +129,7 @@ def pack_lm_head(wte):
     Vp = -(-V // 64) * 64
     lib = _lib.load()
     buf = torch.zeros(lib.gptmi_packed_weight_bytes(Vp, H), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_pack_weight(wte.data_ptr(), buf.data_ptr(), V, H, _lib.GPTMI_W_NK,
                                    _dtype_code(wte, "pack_lm_head"), _stream())
     _lib.check(rc, "pack_lm_head")
@@ -152,7 +173,7 @@ def fused_embeddings(x, wte, wpe, dropout_prob=0.0):
     _maybe_check_ids(x, V)
     z = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_embed(x.data_ptr(), wte.data_ptr(), wpe.data_ptr(), z.data_ptr(), B, L, V,
                              P, H, float(dropout_prob), 1337, _dtype_code(wte, "fused_embeddings"),
                              _stream())
@@ -185,7 +206,7 @@ def fused_embeddings_layer_norm(x, wte, wpe, weight, bias):
     emb = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     out = torch.empty((B * L, H), device=dev, dtype=wte.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_embed_layernorm(x.data_ptr(), wte.data_ptr(), wpe.data_ptr(),
                                        weight.data_ptr(), bias.data_ptr(), emb.data_ptr(),
                                        out.data_ptr(), B, L, V, P, H, 1e-5,
@@ -209,7 +230,7 @@ def fused_layer_norm(x, weight, bias):
     M = x.numel() // H
     z = torch.empty(x.shape, device=dev, dtype=x.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_layernorm(x.data_ptr(), weight.data_ptr(), bias.data_ptr(), z.data_ptr(), M,
                                  H, 1e-5, _dtype_code(x, "fused_layer_norm"), _stream())
     _lib.check(rc, "fused_layer_norm")
@@ -225,7 +246,7 @@ def fused_softmax(x):
     M = x.numel() // H
     z = torch.empty(x.shape, device=dev, dtype=x.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_softmax(x.data_ptr(), z.data_ptr(), M, H, _dtype_code(x, "fused_softmax"),
                                _stream())
     _lib.check(rc, "fused_softmax")
@@ -243,7 +264,7 @@ def _linear(x2d, weight, bias, residual, z, gelu, dropout_prob, wlayout, what):
     lib = _lib.load()
     ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, wlayout)
     ws = _workspace(ws_bytes, dev)
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_linear(x2d.data_ptr(), weight.data_ptr(), _ptr(bias), _ptr(residual),
                               z.data_ptr(), M, N, K, int(bool(gelu)), float(dropout_prob), 1337,
                               wlayout, _ptr(ws), ws_bytes, code, _stream())
@@ -335,7 +356,7 @@ def matmul_and_split_qkv(x, weight, bias, num_heads):
     wl = _wlayout(weight, _lib.GPTMI_W_KN)
     ws_bytes = lib.gptmi_linear_workspace_bytes(M, N, K, code, wl)
     ws = _workspace(ws_bytes, dev)
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_linear_qkv(x.data_ptr(), weight.data_ptr(), _ptr(bias), q.data_ptr(),
                                   k.data_ptr(), v.data_ptr(), batch_size, seqlen, num_heads,
                                   head_size, K, wl, _ptr(ws), ws_bytes, code, _stream())
@@ -379,7 +400,7 @@ def layer_norm_ffn(x, ln_weight, ln_bias, weight, bias=None, add_gelu=False):
     M = x.numel() // K
     z = torch.empty((*x.shape[:-1], N), device=dev, dtype=x.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_layernorm_linear(x.data_ptr(), ln_weight.data_ptr(), ln_bias.data_ptr(),
                                         1e-5, weight.data_ptr(), _ptr(bias), z.data_ptr(), M, N, K,
                                         int(bool(add_gelu)), _lib.GPTMI_F16, _stream())
@@ -402,7 +423,7 @@ def layer_norm_matmul_and_split_qkv(x, ln_weight, ln_bias, weight, bias, num_hea
     k = torch.empty(shape, device=dev, dtype=x.dtype)
     v = torch.empty(shape, device=dev, dtype=x.dtype)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_layernorm_linear_qkv(x.data_ptr(), ln_weight.data_ptr(), ln_bias.data_ptr(),
                                             1e-5, weight.data_ptr(), _ptr(bias), q.data_ptr(),
                                             k.data_ptr(), v.data_ptr(), batch_size, seqlen,
@@ -446,7 +467,7 @@ def _flash(q, k, v, scale, dropout_prob, merged_heads_layout, dev, code):
         buf = torch.empty((B, N, Lq, H), device=dev, dtype=q.dtype)
         layout = _lib.GPTMI_O_BNLD
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _device(dev):
         rc = lib.gptmi_flash_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), buf.data_ptr(), B, N,
                                   Lq, Lk, H, scale, float(dropout_prob), 1337, layout, code,
                                   _stream())
