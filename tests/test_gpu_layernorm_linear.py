@@ -68,6 +68,7 @@ def operands(M, H, N, seed):
     (40, 1280, 1280, False, True),   # large: five chunks per lane (the eight-chunk variant)
     (32, 1600, 6400, True, True),    # XL: seven chunks per lane, the widest panel that fits
     (5, 64, 64, False, False),
+    (5000, 768, 768, False, True),   # 157 row tiles, the last with 8 rows (far beyond where the model uses it)
 ])
 def test_layer_norm_ffn(K, gpu_device, M, H, N, gelu, bias):
     x, ln_w, ln_b, w, b = operands(M, H, N, seed=M + H + N)
