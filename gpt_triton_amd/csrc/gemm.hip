@@ -936,7 +936,9 @@ __global__ __launch_bounds__(WM * WN * 64, WPE) void gemm_kernel(
     if (ln.lpr == 32) GPTMI_LN_ROWS(32);
     else GPTMI_LN_ROWS(64);
 #undef GPTMI_LN_ROWS
-    // panel written, the first weight k-tiles landed (the compiler's barrier waits for both)
+    // the first weight k-tiles have landed (their loads are older than the rows' loads, which
+    // the arithmetic above waited for; said explicitly all the same), the panel is written
+    wait_vmcnt<0>();
     __syncthreads();
   } else {
     // tile 0 must have landed; up to NST-1 younger tiles stay in flight
